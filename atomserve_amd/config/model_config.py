@@ -457,3 +457,192 @@ class KoravikConfig:
         if self.loop:
             raw["loop"] = {"start": self.loop_start, "stop": self.loop_stop, "times": self.loop_times}
         return raw
+
+
+# ---- Mumizen ------------------------------------------------------------------------------------------
+
+
+@dataclass(frozen=True)
+class MumizenDecay:
+    """A linear-attention mixer with a fixed decay per head ("lightning" or "retention")."""
+
+    heads: int
+    dim: int  # width of a query/key head
+    vdim: int  # width of a value head
+    decay: tuple  # per head
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "MumizenDecay":
+        decay = _need(raw, "decay", where)
+        return cls(int(_need(raw, "heads", where)), int(_need(raw, "dim", where)), int(_need(raw, "vdim", where)),
+                   tuple(float(d) for d in decay))  # fmt: skip
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "decay": list(self.decay)}
+
+
+@dataclass(frozen=True)
+class MumizenLatent:
+    """An attention through a latent.  kv_from >= 0: the layer has no latent of its own and reads that layer's."""
+
+    heads: int
+    dim: int  # coordinates of a query/key head that are not rotated
+    rot_dim: int  # and those that are
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    rot_base: float
+    scaling: object  # None, or (factor, original, fast, slow)
+    kv_from: int = -1
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "MumizenLatent":
+        rot = raw.get("rot") or {}
+        rot_dim = int(_need(raw, "rot_dim", where))
+        if rot_dim and int(_need(rot, "dims", where + "rot.")) != rot_dim:
+            raise ConfigError(f"{where}rot.dims must equal rot_dim")
+        scaling = rot.get("scaling")
+        if scaling:
+            scaling = tuple(float(_need(scaling, k, where + "rot.scaling.")) for k in ("factor", "original", "fast", "slow"))
+        return cls(
+            heads=int(_need(raw, "heads", where)),
+            dim=int(_need(raw, "dim", where)),
+            rot_dim=rot_dim,
+            vdim=int(_need(raw, "vdim", where)),
+            q_rank=int(_need(raw, "q_rank", where)),
+            kv_rank=int(_need(raw, "kv_rank", where)),
+            scale=float(_need(raw, "scale", where)),
+            rot_base=float(_need(rot, "base", where + "rot.")) if rot_dim else 1.0,
+            scaling=scaling or None,
+            kv_from=int(raw["kv_from"]) if raw.get("kv_from") is not None else -1,
+        )
+
+    def to_dict(self) -> dict:
+        raw = {"heads": self.heads, "dim": self.dim, "rot_dim": self.rot_dim, "vdim": self.vdim, "q_rank": self.q_rank,
+               "kv_rank": self.kv_rank, "scale": self.scale}  # fmt: skip
+        if self.rot_dim:
+            raw["rot"] = {"dims": self.rot_dim, "base": self.rot_base}
+            if self.scaling:
+                raw["rot"]["scaling"] = dict(zip(("factor", "original", "fast", "slow"), self.scaling))
+        if self.kv_from >= 0:
+            raw["kv_from"] = self.kv_from
+        return raw
+
+
+@dataclass(frozen=True)
+class MumizenFeedForward:
+    kind: str  # "dense" or "moe"
+    ff: int  # width inside the feed-forward (of one expert for "moe")
+    limit: float
+    experts: int = 0
+    top: int = 0
+    shared_ff: int = 0
+    shared_limit: float = 0.0
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "MumizenFeedForward":
+        kind = _need(raw, "kind", where)
+        if kind == "dense":
+            return cls("dense", int(_need(raw, "ff", where)), float(_need(raw, "limit", where)))
+        if kind == "moe":
+            expert, router = _need(raw, "expert", where), _need(raw, "router", where)
+            shared = raw.get("shared") or {}
+            return cls("moe", int(_need(expert, "ff", where + "expert.")), float(_need(expert, "limit", where + "expert.")),
+                       int(_need(router, "experts", where + "router.")), int(_need(router, "top", where + "router.")),
+                       int(shared.get("ff", 0)), float(_need(shared, "limit", where + "shared.")) if shared.get("ff") else 0.0)  # fmt: skip
+        raise ConfigError(f"{where}kind={kind!r} is not supported ('dense' or 'moe')")
+
+    def to_dict(self) -> dict:
+        if self.kind == "dense":
+            return {"kind": "dense", "ff": self.ff, "limit": self.limit}
+        raw = {"kind": "moe", "expert": {"ff": self.ff, "limit": self.limit}, "router": {"experts": self.experts, "top": self.top}}
+        if self.shared_ff:
+            raw["shared"] = {"ff": self.shared_ff, "limit": self.shared_limit}
+        return raw
+
+
+@dataclass(frozen=True)
+class MumizenLayer:
+    type: str  # "lightning", "retention" or "latent_attention"
+    mixer: object  # MumizenDecay or MumizenLatent
+    mlp: object  # MumizenFeedForward or None
+
+
+@dataclass(frozen=True)
+class MumizenConfig:
+    """A Mumizen decoder: pre-norm layers with norms in groups, a token shift before every mixer and an average over
+    the results of all layers so far after every layer; mixers are linear attentions with fixed decays or attentions
+    through a latent (which may read an earlier layer's), feed-forwards dense or routed with a shared expert."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    norm_groups: int
+    layers: tuple  # of MumizenLayer
+
+    architecture = "Mumizen"
+    MIXERS = ("lightning", "retention", "latent_attention")
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "MumizenConfig":
+        _require(raw, ["vocab", "width", "layers", "norm"])
+        layers = []
+        for i, entry in enumerate(raw["layers"]):
+            where = f"layers[{i}]."
+            kind = _need(entry, "type", where)
+            if kind in ("lightning", "retention"):
+                mixer = MumizenDecay.from_dict(_need(entry, "mixer", where), where + "mixer.")
+            elif kind == "latent_attention":
+                mixer = MumizenLatent.from_dict(_need(entry, "mixer", where), where + "mixer.")
+            else:
+                raise ConfigError(f"{where}type={kind!r} is not supported (one of {', '.join(cls.MIXERS)})")
+            mlp = entry.get("mlp")
+            layers.append(MumizenLayer(kind, mixer, None if mlp is None else MumizenFeedForward.from_dict(mlp, where + "mlp.")))
+        cfg = cls(
+            vocab_size=int(raw["vocab"]),
+            hidden_size=int(raw["width"]),
+            norm_eps=float(_need(raw["norm"], "eps", "norm.")),
+            norm_groups=int(raw["norm"].get("groups", 1)),
+            layers=tuple(layers),
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size < 1 or self.hidden_size < 1 or not self.layers:
+            raise ConfigError("vocab, width and the number of layers must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        if self.norm_groups < 1 or self.hidden_size % self.norm_groups:
+            raise ConfigError(f"norm.groups {self.norm_groups} does not divide the width {self.hidden_size}")
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            if layer.type == "latent_attention":
+                if min(m.heads, m.dim, m.vdim, m.q_rank, m.kv_rank) < 1 or m.rot_dim < 0 or m.rot_dim % 2:
+                    raise ConfigError(f"layers[{i}]: sizes must be positive and rot_dim even")
+                if m.rot_dim and not m.rot_base > 1:
+                    raise ConfigError(f"layers[{i}]: rot.base must exceed 1")
+                if m.kv_from >= 0:
+                    src = self.layers[m.kv_from] if m.kv_from < i else None
+                    if src is None or src.type != "latent_attention" or src.mixer.kv_from >= 0:
+                        raise ConfigError(f"layers[{i}]: kv_from names an earlier latent-attention layer with a latent of its own")
+                    s = src.mixer
+                    if (s.kv_rank, s.rot_dim, s.rot_base, s.scaling) != (m.kv_rank, m.rot_dim, m.rot_base, m.scaling):
+                        raise ConfigError(f"layers[{i}]: kv_rank, rot_dim and rotation must equal those of layer {m.kv_from}")
+            else:
+                if min(m.heads, m.dim, m.vdim) < 1 or len(m.decay) != m.heads:
+                    raise ConfigError(f"layers[{i}]: sizes must be positive, with one decay per head")
+                if any(not 0.0 <= d <= 1.0 for d in m.decay):
+                    raise ConfigError(f"layers[{i}]: decays lie between 0 and 1")
+            f = layer.mlp
+            if f is not None and (f.ff < 1 or not f.limit > 0 or (f.kind == "moe" and not 1 <= f.top <= f.experts)
+                                  or f.shared_ff < 0 or (f.shared_ff and not f.shared_limit > 0)):  # fmt: skip
+                raise ConfigError(f"layers[{i}].mlp: sizes and limits must be positive and top at most the number of experts")
+
+    def to_dict(self) -> dict:
+        """The config.json that `from_dict` reads back to this object."""
+        layers = [{"type": layer.type, "mixer": layer.mixer.to_dict(), "mlp": None if layer.mlp is None else layer.mlp.to_dict()}
+                  for layer in self.layers]  # fmt: skip
+        return {"architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+                "norm": {"eps": self.norm_eps, "groups": self.norm_groups}, "layers": layers}  # fmt: skip

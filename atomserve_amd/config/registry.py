@@ -23,7 +23,7 @@ class Architecture:
     checkpoint_shapes: typed configuration -> {checkpoint name: (shape, role)}, in the order in which
                     random weights are drawn; roles: "matrix", "vector" (gains around 1), "bias" and
                     "log_rate" (small values around 0), "near_identity" (a square matrix around the
-                    identity), "expert_table:<experts>" (int32 rows of distinct expert numbers)
+                    identity), "fraction" (values between 0 and 1), "depth_weights" (mostly on the last entry), "expert_table:<experts>" (int32 rows of distinct expert numbers)
     ignored:        typed configuration -> checkpoint names that may be present and unused
     """
 
@@ -79,4 +79,5 @@ def _load_builtin() -> None:
     # Imported lazily: the model modules import parts, which import this package.
     import atomserve_amd.models.dozusun  # noqa: F401
     import atomserve_amd.models.koravik  # noqa: F401
+    import atomserve_amd.models.mumizen  # noqa: F401
     import atomserve_amd.models.qwen3  # noqa: F401

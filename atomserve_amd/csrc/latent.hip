@@ -1,0 +1,204 @@
+// Attention through a latent: keys and values of all heads are matrices times one cached vector c [kv_rank] per
+// token, beside one rotated key part k_r [rot_dim] that all heads share.  With k_h = U_h c and v_h = V_h c,
+//
+//   q_h . k_h = (U_h^T q_h) . c          and          sum_j p_j v_h(j) = V_h (sum_j p_j c_j),
+//
+// so the attention itself runs over one kv head whose keys are [c | k_r] and whose values are c, with queries
+// [U_h^T q_h | rotated part of q_h]: the paged attention kernels of this package as they are.  Here are the steps
+// around them:
+//
+//   rows_rms_norm     a plain RMS norm of columns of a product's result (the latent of the queries)
+//   latent_kv_store   norm of c, rotation of k_r, [c | k_r] into the key pages and c into the value pages
+//   latent_q_absorb   q [T, H, D + R] -> [U_h^T q_h | rotate(q_h[D:])], zeros up to the pages' width
+//   latent_v_expand   heads [T, H, width] (their first kv_rank coordinates) -> V_h heads, times sigmoid(gate)
+//
+// Norms, the rotation and every sum are fp32; an output is one chain of multiply-adds in a fixed order.
+#include "common.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void rows_rms_norm_kernel(const T* __restrict__ proj, int ld, int off, int n,
+                                                            const float* __restrict__ gain, float eps,
+                                                            T* __restrict__ out) {
+  __shared__ float red[17];
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * ld + off;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = to_f32(row[i]); ss = fmaf(v, v, ss); }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) out[(size_t)t * n + i] = from_f32<T>(to_f32(row[i]) * inv * gain[i]);
+}
+
+extern "C" int as_rows_rms_norm(const void* proj, int dtype, int ld, int off, int n, const float* gain, float eps,
+                                void* out, int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (n <= 0 || off < 0 || off + n > ld) return AS_BAD_SHAPE;
+  if (dtype == DT_F32) rows_rms_norm_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)proj, ld, off, n, gain, eps, (float*)out);
+  else if (dtype == DT_BF16) rows_rms_norm_kernel<bf16><<<num_tokens, 256, 0, stream>>>((const bf16*)proj, ld, off, n, gain, eps, (bf16*)out);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// proj[t, off .. off + rank) is the latent before its norm, the next `rot` columns the shared key part before its
+// rotation; cos_sin [T, rot/2, 2] fp32.  k_pages [pages, 1, bs, width], v_pages [pages, 1, width, bs]; slots[t] < 0:
+// nothing is stored.  What is not finite is stored as zero; the pages' columns beyond what is stored get zeros.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_kv_store_kernel(const T* __restrict__ proj, int ld, int off, int rank,
+                                                              int rot, const float* __restrict__ gain, float eps,
+                                                              const float* __restrict__ cos_sin,
+                                                              const int* __restrict__ slots, T* __restrict__ k_pages,
+                                                              T* __restrict__ v_pages, int bs, int width) {
+  __shared__ float red[17];
+  const int t = blockIdx.x;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  const T* row = proj + (size_t)t * ld + off;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) { const float v = to_f32(row[i]); ss = fmaf(v, v, ss); }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)rank + eps);
+  const int page = slot / bs, in_page = slot % bs;
+  T* kd = k_pages + ((size_t)page * bs + in_page) * width;
+  T* vd = v_pages + (size_t)page * width * bs + in_page;
+  const int half = rot / 2;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float key = 0.f, value = 0.f;
+    if (i < rank) {
+      key = value = to_f32(row[i]) * inv * gain[i];
+    } else if (i < rank + rot) {
+      const int j = i - rank, p = j < half ? j : j - half;
+      const float c = cos_sin[((size_t)t * half + p) * 2], s = cos_sin[((size_t)t * half + p) * 2 + 1];
+      const float u = to_f32(row[rank + p]), v = to_f32(row[rank + half + p]);
+      key = j < half ? u * c - v * s : v * c + u * s;
+    }
+    kd[i] = finite_or_zero(from_f32<T>(key));
+    vd[(size_t)i * bs] = finite_or_zero(from_f32<T>(value));
+  }
+}
+
+extern "C" int as_latent_kv_store(const void* proj, int dtype, int ld, int off, int rank, int rot, const float* gain,
+                                  float eps, const float* cos_sin, const int* slots, void* k_pages, void* v_pages,
+                                  int bs, int width, int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (rank <= 0 || rot < 0 || rot % 2 || rank + rot > width || off < 0 || off + rank + rot > ld || bs <= 0) return AS_BAD_SHAPE;
+  if (rot > 0 && !cos_sin) return AS_BAD_SHAPE;
+  if (dtype == DT_F32)
+    latent_kv_store_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)proj, ld, off, rank, rot, gain, eps, cos_sin, slots,
+                                                                 (float*)k_pages, (float*)v_pages, bs, width);
+  else if (dtype == DT_BF16)
+    latent_kv_store_kernel<bf16><<<num_tokens, 256, 0, stream>>>((const bf16*)proj, ld, off, rank, rot, gain, eps, cos_sin, slots,
+                                                                (bf16*)k_pages, (bf16*)v_pages, bs, width);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// q [T, H, D + R]; uk [H * D, rank] (row h D + d: what coordinate d of head h's keys reads of the latent).
+// out [T, H, width]: out[t, h, r] = sum_d q[t, h, d] uk[h D + d, r] for r < rank, then the R rotated coordinates
+// of q, then zeros.  grid (token tiles of ABSORB_TOKENS, heads).
+#define ABSORB_TOKENS 8
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_q_absorb_kernel(const T* __restrict__ q, const T* __restrict__ uk, int H,
+                                                              int D, int R, int rank, const float* __restrict__ cos_sin,
+                                                              T* __restrict__ out, int width, int num_tokens) {
+  extern __shared__ float qs[];  // [ABSORB_TOKENS][D]
+  const int t0 = blockIdx.x * ABSORB_TOKENS, h = blockIdx.y;
+  const int nt = min(ABSORB_TOKENS, num_tokens - t0);
+  for (int i = threadIdx.x; i < ABSORB_TOKENS * D; i += blockDim.x) {
+    const int tq = i / D, d = i % D;
+    qs[i] = tq < nt ? to_f32(q[((size_t)(t0 + tq) * H + h) * (D + R) + d]) : 0.f;
+  }
+  __syncthreads();
+  const T* w = uk + (size_t)h * D * rank;
+  for (int r = threadIdx.x; r < rank; r += blockDim.x) {
+    float acc[ABSORB_TOKENS];
+#pragma unroll
+    for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = 0.f;
+    for (int d = 0; d < D; ++d) {
+      const float wv = to_f32(w[(size_t)d * rank + r]);
+#pragma unroll
+      for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = fmaf(qs[tq * D + d], wv, acc[tq]);
+    }
+    for (int tq = 0; tq < nt; ++tq) out[((size_t)(t0 + tq) * H + h) * width + r] = from_f32<T>(acc[tq]);
+  }
+  const int half = R / 2, tail = width - rank;
+  for (int i = threadIdx.x; i < nt * tail; i += blockDim.x) {
+    const int tq = i / tail, j = i % tail, t = t0 + tq;
+    float v = 0.f;
+    if (j < R) {
+      const int p = j < half ? j : j - half;
+      const T* qr = q + ((size_t)t * H + h) * (D + R) + D;
+      const float c = cos_sin[((size_t)t * half + p) * 2], s = cos_sin[((size_t)t * half + p) * 2 + 1];
+      const float a = to_f32(qr[p]), b = to_f32(qr[half + p]);
+      v = j < half ? a * c - b * s : b * c + a * s;
+    }
+    out[((size_t)t * H + h) * width + rank + j] = from_f32<T>(v);
+  }
+}
+
+extern "C" int as_latent_q_absorb(const void* q, const void* uk, int dtype, int H, int D, int R, int rank,
+                                  const float* cos_sin, void* out, int width, int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (H <= 0 || H > 65535 || D <= 0 || R < 0 || R % 2 || rank <= 0 || rank + R > width || D > 1024) return AS_BAD_SHAPE;
+  if (R > 0 && !cos_sin) return AS_BAD_SHAPE;
+  dim3 grid((num_tokens + ABSORB_TOKENS - 1) / ABSORB_TOKENS, H);
+  const size_t lds = (size_t)ABSORB_TOKENS * D * sizeof(float);
+  if (dtype == DT_F32)
+    latent_q_absorb_kernel<float><<<grid, 256, lds, stream>>>((const float*)q, (const float*)uk, H, D, R, rank, cos_sin, (float*)out, width, num_tokens);
+  else if (dtype == DT_BF16)
+    latent_q_absorb_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)uk, H, D, R, rank, cos_sin, (bf16*)out, width, num_tokens);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// heads [T, H, width]: what the attention over the latent left per head (its first `rank` coordinates count).
+// uv_t [H, rank, E]: head h's value matrix, transposed.  out[t, h E + e] = (sum_r heads[t, h, r] uv_t[h, r, e]) *
+// sigmoid(gate[t, g_off + h E + e]) (gate null: no gate).  grid (token tiles of ABSORB_TOKENS, heads).
+template <typename T>
+__global__ __launch_bounds__(256) void latent_v_expand_kernel(const T* __restrict__ heads, const T* __restrict__ uv_t,
+                                                              int H, int E, int rank, int width,
+                                                              const T* __restrict__ gate, int ld, int g_off,
+                                                              T* __restrict__ out, int num_tokens) {
+  extern __shared__ float os[];  // [ABSORB_TOKENS][rank]
+  const int t0 = blockIdx.x * ABSORB_TOKENS, h = blockIdx.y;
+  const int nt = min(ABSORB_TOKENS, num_tokens - t0);
+  for (int i = threadIdx.x; i < ABSORB_TOKENS * rank; i += blockDim.x) {
+    const int tq = i / rank, r = i % rank;
+    os[i] = tq < nt ? to_f32(heads[((size_t)(t0 + tq) * H + h) * width + r]) : 0.f;
+  }
+  __syncthreads();
+  const T* w = uv_t + (size_t)h * rank * E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    float acc[ABSORB_TOKENS];
+#pragma unroll
+    for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = 0.f;
+    for (int r = 0; r < rank; ++r) {
+      const float wv = to_f32(w[(size_t)r * E + e]);
+#pragma unroll
+      for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = fmaf(os[tq * rank + r], wv, acc[tq]);
+    }
+    for (int tq = 0; tq < nt; ++tq) {
+      const size_t t = t0 + tq;
+      float v = acc[tq];
+      if (gate) {
+        v = to_f32(from_f32<T>(v));  // the head's value as it would be stored
+        v *= 1.0f / (1.0f + expf(-to_f32(gate[t * ld + g_off + h * E + e])));
+      }
+      out[(t * H + h) * E + e] = from_f32<T>(v);
+    }
+  }
+}
+
+extern "C" int as_latent_v_expand(const void* heads, const void* uv_t, int dtype, int H, int E, int rank, int width,
+                                  const void* gate, int ld, int g_off, void* out, int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (H <= 0 || H > 65535 || E <= 0 || rank <= 0 || rank > width || rank > 4096) return AS_BAD_SHAPE;
+  dim3 grid((num_tokens + ABSORB_TOKENS - 1) / ABSORB_TOKENS, H);
+  const size_t lds = (size_t)ABSORB_TOKENS * rank * sizeof(float);
+  if (dtype == DT_F32)
+    latent_v_expand_kernel<float><<<grid, 256, lds, stream>>>((const float*)heads, (const float*)uv_t, H, E, rank, width, (const float*)gate, ld, g_off, (float*)out, num_tokens);
+  else if (dtype == DT_BF16)
+    latent_v_expand_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)heads, (const bf16*)uv_t, H, E, rank, width, (const bf16*)gate, ld, g_off, (bf16*)out, num_tokens);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}

@@ -75,8 +75,9 @@ __global__ __launch_bounds__(1024) void moe_route_table_kernel(const int* __rest
 }
 
 // ---- a router that scores every expert ---------------------------------------------------------------
-// z = router h in fp32 (router [experts, K], h [T, K], both T-typed), s = sigmoid(z); a token's `top` experts are
-// those with the largest s (of equal ones the lower number first); their weights are s / (sum of the chosen + 1e-20).
+// z = router h (+ bias [experts] fp32) in fp32 (router [experts, K], h [T, K], both T-typed).  mode 0: s = sigmoid(z); a
+// token's `top` experts are those with the largest s (of equal ones the lower number first); their weights are
+// s / (sum of the chosen + 1e-20).  mode 1: the experts with the largest z, weighing the softmax over the chosen z alone.
 // pair_expert, pair_weight [T * top].  A workgroup per token: its waves take the experts four at a time, a lane 16 bytes
 // of the token's row and of the four router rows at a time (the rows stream once, coalesced), the sums meet by lane swaps
 // and the scores in LDS, where the first wave makes the choice.
@@ -98,7 +99,8 @@ template <> struct RoutePiece<bf16> {
 };
 
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(const T* __restrict__ h, const T* __restrict__ router,
+__global__ __launch_bounds__(256) void moe_route_scores_kernel(const T* __restrict__ h, const T* __restrict__ router,
+                                                                const float* __restrict__ bias, int mode,
                                                                 int K, int experts, int top, int num_tokens,
                                                                 int* __restrict__ pair_expert,
                                                                 float* __restrict__ pair_weight) {
@@ -132,17 +134,20 @@ __global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(const T* __restr
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float zs = wave_sum(z[j]);
-      if (lane == 0 && e0 + j < experts) scores[e0 + j] = 1.0f / (1.0f + expf(-zs));
+      float zs = wave_sum(z[j]);
+      if (lane == 0 && e0 + j < experts) {
+        if (bias) zs += bias[e0 + j];
+        scores[e0 + j] = mode == 1 ? zs : 1.0f / (1.0f + expf(-zs));
+      }
     }
   }
   __syncthreads();
   if (wave) return;
   float* mine = scores;
-  float total = 0.f, my_score = 0.f;
+  float total = 0.f, my_score = 0.f, largest = 0.f;
   int my_expert = 0;
   for (int j = 0; j < top; ++j) {
-    float best = -1.f;
+    float best = -INFINITY;
     int at = 0x7fffffff;
     for (int e = lane; e < experts; e += WAVE) {
       const float v = mine[e];
@@ -155,16 +160,20 @@ __global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(const T* __restr
       if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
     }
     if (at >= experts) { at = 0; best = 0.f; }  // nothing left to choose (scores that are not numbers)
+    if (mode == 1) {  // the first found is the largest: weights are exponentials of the distance to it
+      if (j == 0) largest = best;
+      best = expf(best - largest);
+    }
     if (lane == j % WAVE && j / WAVE == 0) { my_score = best; my_expert = at; }
     if (j >= WAVE && lane == 0) {  // more than 64 experts a token: written as they are found, weighed below
       pair_expert[(size_t)t * top + j] = at;
       pair_weight[(size_t)t * top + j] = best;
     }
     total += best;
-    if (lane == 0) mine[at] = -2.f;
+    if (lane == 0) mine[at] = -INFINITY;
     __builtin_amdgcn_wave_barrier();
   }
-  const float inv = 1.0f / (total + 1e-20f);
+  const float inv = 1.0f / (total + (mode == 1 ? 0.f : 1e-20f));
   if (lane < top && lane < WAVE) {
     pair_expert[(size_t)t * top + lane] = my_expert;
     pair_weight[(size_t)t * top + lane] = my_score * inv;
@@ -173,17 +182,18 @@ __global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(const T* __restr
     for (int j = WAVE; j < top; ++j) pair_weight[(size_t)t * top + j] *= inv;
 }
 
-extern "C" int as_moe_route_sigmoid(const void* h, const void* router, int dtype, int K, int experts, int top,
-                                    int num_tokens, int* pair_expert, float* pair_weight, hipStream_t stream) {
+extern "C" int as_moe_route_scores(const void* h, const void* router, const float* bias, int mode, int dtype, int K,
+                                   int experts, int top, int num_tokens, int* pair_expert, float* pair_weight,
+                                   hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
-  if (K <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts) return AS_BAD_SHAPE;
+  if (K <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts || mode < 0 || mode > 1) return AS_BAD_SHAPE;
   const int blocks = num_tokens;
   const size_t lds = (size_t)experts * sizeof(float);
   if (dtype == DT_F32)
-    moe_route_sigmoid_kernel<float><<<blocks, 256, lds, stream>>>((const float*)h, (const float*)router, K, experts, top,
+    moe_route_scores_kernel<float><<<blocks, 256, lds, stream>>>((const float*)h, (const float*)router, bias, mode, K, experts, top,
                                                                   num_tokens, pair_expert, pair_weight);
   else if (dtype == DT_BF16)
-    moe_route_sigmoid_kernel<bf16><<<blocks, 256, lds, stream>>>((const bf16*)h, (const bf16*)router, K, experts, top,
+    moe_route_scores_kernel<bf16><<<blocks, 256, lds, stream>>>((const bf16*)h, (const bf16*)router, bias, mode, K, experts, top,
                                                                  num_tokens, pair_expert, pair_weight);
   else return AS_BAD_DTYPE;
   return launch_status();
@@ -221,12 +231,24 @@ __device__ __forceinline__ bf16x8 row_piece(const bf16* row, int k, int K) {
   return v;
 }
 
+// silu(g) * u, or with limits (limit > 0): g = min(g, limit), u = clamp(u, -limit, limit): g sigmoid(1.702 g) (u + 1)
+#define CLAMPED_GATE_ALPHA 1.702f
+__device__ __forceinline__ float gate_times_up(float g, float u, float limit) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-CLAMPED_GATE_ALPHA * g)) * (u + 1.0f);
+  }
+  return g / (1.0f + expf(-g)) * u;
+}
+
 template <bool GATED, typename OutT, bool RELU2 = false>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restrict__ a, int a_div,
                                                             const bf16* __restrict__ w, int N, int K,
                                                             const int* __restrict__ order,
                                                             const int* __restrict__ tiles,
-                                                            const int* __restrict__ counts, OutT* __restrict__ out) {
+                                                            const int* __restrict__ counts, OutT* __restrict__ out,
+                                                            float limit) {
   constexpr int WROWS = GATED ? 2 * MOE_STRIP : MOE_STRIP;  // weight rows of a round: the strip's, then their up rows
   constexpr int WLOADS = WROWS * (MOE_KC / 8) / 256;        // 16-byte pieces of them per thread
   __shared__ __attribute__((aligned(16))) bf16 acts[MOE_TILE][MOE_KC + 8];
@@ -328,7 +350,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(const bf16* __restri
       float v = acc[ct][i];
       if (GATED) {
         const float g = to_f32((bf16)acc[ct][i]), u = to_f32((bf16)acc_up[ct][i]);  // the two products rounded as if stored
-        v = g / (1.0f + expf(-g)) * u;
+        v = gate_times_up(g, u, limit);
       }
       if (RELU2) {
         const float u = fmaxf(to_f32((bf16)v), 0.f);  // the product rounded as if stored
@@ -346,7 +368,8 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(const float* __restri
                                                            const float* __restrict__ w, int N, int K,
                                                            const int* __restrict__ order,
                                                            const int* __restrict__ tiles,
-                                                           const int* __restrict__ counts, float* __restrict__ out) {
+                                                           const int* __restrict__ counts, float* __restrict__ out,
+                                                           float limit) {
   const int tile = blockIdx.y;
   if (tile >= counts[0]) return;
   const int e = tiles[3 * tile], at = tiles[3 * tile + 1], cnt = tiles[3 * tile + 2];
@@ -379,7 +402,7 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(const float* __restri
     for (int i = 0; i < 4; ++i) {
       if (pairs[i] < 0) continue;
       float v = acc[i];
-      if (GATED) v = v / (1.0f + expf(-v)) * acc_up[i];
+      if (GATED) v = gate_times_up(v, acc_up[i], limit);
       if (RELU2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
       out[(size_t)pairs[i] * N + n] = v;
     }
@@ -388,31 +411,32 @@ __global__ __launch_bounds__(256) void moe_gemm_f32_kernel(const float* __restri
 
 // out_dtype: DT_BF16 or DT_F32 for the bf16 product's results (fp32 where several experts' outputs
 // are still to be added up); the fp32 product writes fp32.
-// gated: 0: the product; 1: silu(gate) * up; 2: relu(product)^2 (an expert without a gate).
+// gated: 0: the product; 1: act(gate) * up (limit 0: silu(gate) * up; > 0: the gated activation with limits);
+// 2: relu(product)^2 (an expert without a gate).
 extern "C" int as_moe_gemm(const void* a, int dtype, int a_div, const void* w, int N, int K, int gated, const int* order,
-                           const int* tiles, const int* counts, int max_tiles, void* out, int out_dtype,
+                           const int* tiles, const int* counts, int max_tiles, void* out, int out_dtype, float limit,
                            hipStream_t stream) {
   if (max_tiles <= 0) return AS_OK;
   if (N <= 0 || K <= 0 || a_div <= 0 || max_tiles > 65535) return AS_BAD_SHAPE;
   dim3 grid((N + MOE_STRIP - 1) / MOE_STRIP, max_tiles);
   if (dtype == DT_F32) {
     if (out_dtype != DT_F32) return AS_BAD_DTYPE;
-    if (gated == 2) moe_gemm_f32_kernel<false, true><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out);
-    else if (gated) moe_gemm_f32_kernel<true><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out);
-    else moe_gemm_f32_kernel<false><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out);
+    if (gated == 2) moe_gemm_f32_kernel<false, true><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out, limit);
+    else if (gated) moe_gemm_f32_kernel<true><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out, limit);
+    else moe_gemm_f32_kernel<false><<<grid, 256, 0, stream>>>((const float*)a, a_div, (const float*)w, N, K, order, tiles, counts, (float*)out, limit);
     return launch_status();
   }
   if (dtype != DT_BF16) return AS_BAD_DTYPE;
   if (gated == 2) {
     if (out_dtype != DT_BF16) return AS_BAD_DTYPE;
-    moe_gemm_bf16_kernel<false, bf16, true><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out);
+    moe_gemm_bf16_kernel<false, bf16, true><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out, limit);
   } else if (gated) {
     if (out_dtype != DT_BF16) return AS_BAD_DTYPE;
-    moe_gemm_bf16_kernel<true, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out);
+    moe_gemm_bf16_kernel<true, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out, limit);
   } else if (out_dtype == DT_BF16) {
-    moe_gemm_bf16_kernel<false, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out);
+    moe_gemm_bf16_kernel<false, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (bf16*)out, limit);
   } else if (out_dtype == DT_F32) {
-    moe_gemm_bf16_kernel<false, float><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (float*)out);
+    moe_gemm_bf16_kernel<false, float><<<grid, 256, 0, stream>>>((const bf16*)a, a_div, (const bf16*)w, N, K, order, tiles, counts, (float*)out, limit);
   } else {
     return AS_BAD_DTYPE;
   }

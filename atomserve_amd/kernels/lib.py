@@ -36,9 +36,19 @@ SIGNATURES = {
     "as_rglru_gates": ("recurrent", [P, I, I, P, P, P, P, P, I, F, P, P, I, P]),
     "as_rglru_scan": ("recurrent", [P, P, I, P, I, I, I, P, I, F, P, P, P, P, P, I, P, I, I, I, P]),
     "as_moe_route_table": ("moe", [P, P, I, I, I, I, P, P, P, I, P]),
-    "as_moe_gemm": ("moe", [P, I, I, P, I, I, I, P, P, P, I, P, I, P]),
+    "as_moe_gemm": ("moe", [P, I, I, P, I, I, I, P, P, P, I, P, I, F, P]),
     "as_moe_combine": ("moe", [P, I, F, I, P, I, I, P, P, P]),
-    "as_moe_route_sigmoid": ("moe", [P, P, I, I, I, I, I, P, P, P]),
+    "as_moe_route_scores": ("moe", [P, P, P, I, I, I, I, I, I, P, P, P]),
+    "as_group_norm": ("layer_ops", [P, P, P, P, F, I, P, I, I, I, I, P]),
+    "as_group_norm_shift": ("layer_ops", [P, P, P, F, I, P, P, P, P, P, P, P, I, I, I, I, P]),
+    "as_depth_average": ("layer_ops", [P, P, I, P, P, I, c_longlong, P]),
+    "as_clamped_gate": ("layer_ops", [P, P, I, I, I, F, F, P]),
+    "as_decay_scan": ("linear_attention", [P, I, I, I, I, I, I, I, I, I, F, P, P, P, P, P, P, I, P, I, P]),
+    "as_decay_finish": ("linear_attention", [P, I, I, F, P, P, I, I, I, I, P, I, P]),
+    "as_rows_rms_norm": ("latent", [P, I, I, I, I, P, F, P, I, P]),
+    "as_latent_kv_store": ("latent", [P, I, I, I, I, I, P, F, P, P, P, P, I, I, I, P]),
+    "as_latent_q_absorb": ("latent", [P, P, I, I, I, I, I, P, P, I, I, P]),
+    "as_latent_v_expand": ("latent", [P, P, I, I, I, I, I, P, I, I, P, I, P]),
     "as_attn_headmix_mfma": ("attention_mix", [P, P, P, P, I, I, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, P, P, P]),
     "as_attn_headmix": ("attention_mix", [P, P, P, I, P, I, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P]),
     "as_attn_single_query": ("attention", [P, P, P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),

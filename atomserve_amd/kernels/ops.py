@@ -1456,27 +1456,43 @@ def moe_route_sigmoid(h, router, top: int) -> ExpertRoute:
     """Routes by a router's scores: z = router h in fp32, s = sigmoid(z), a token's `top` experts those with the
     largest s, weighing s / (their sum + 1e-20).  h [T, K], router [experts, K] of one dtype.  The route carries
     `pair_weight` fp32 [T * top] for `moe_combine`."""
+    return moe_route_scores(h, router, top, "sigmoid")
+
+
+ROUTER_SCORES = {"sigmoid": 0, "softmax_of_chosen": 1}
+
+
+def moe_route_scores(h, router, top: int, score: str, bias=None) -> ExpertRoute:
+    """Routes by a router's logits z = router h + bias in fp32 (bias fp32 [experts] or None).  score "sigmoid": the
+    `top` largest sigmoid(z), weighing s / (their sum + 1e-20); "softmax_of_chosen": the `top` largest z, weighing the
+    softmax over those z alone.  The route carries `pair_weight` fp32 [T * top] for `moe_combine`."""
     _check(h, "h", (F32, BF16), (None, None))
     T, K = h.shape
     _check(router, "router", h.dtype, (None, K))
     experts = router.shape[0]
+    if score not in ROUTER_SCORES:
+        raise KernelError(f"a router scores by one of {sorted(ROUTER_SCORES)}, not by {score!r}")
+    if bias is not None:
+        _check(bias, "bias", F32, (experts,))
     if not 1 <= top <= experts <= MOE_MAX_EXPERTS:
         raise KernelError(f"routing chooses up to {MOE_MAX_EXPERTS} experts, not {top} of {experts}")
     route = ExpertRoute(T, top, experts, h.device)
     pair_expert = torch.empty(max(T * top, 1), dtype=I32, device=h.device)
     route.pair_weight = torch.empty(max(T * top, 1), dtype=F32, device=h.device)
-    call("as_moe_route_sigmoid", _ptr(h), _ptr(router), _DT[h.dtype], K, experts, top, T, _ptr(pair_expert),
-         _ptr(route.pair_weight), _stream())  # fmt: skip
+    call("as_moe_route_scores", _ptr(h), _ptr(router), _ptr(bias), ROUTER_SCORES[score], _DT[h.dtype], K, experts, top, T,
+         _ptr(pair_expert), _ptr(route.pair_weight), _stream())  # fmt: skip
     call("as_moe_route_table", 0, _ptr(pair_expert), 0, top, experts, T, _ptr(route.order), _ptr(route.tiles),
          _ptr(route.counts), route.max_tiles, _stream())  # fmt: skip
     return route
 
 
-def moe_gemm(a, w, route: ExpertRoute, out, gated: bool, per_token: bool, activation: str = None) -> None:
+def moe_gemm(a, w, route: ExpertRoute, out, gated: bool, per_token: bool, activation: str = None, limit: float = 0.0) -> None:
     """The product of every pair's input with its expert's matrix, w [experts, N_w, K].  per_token: a [T, K] holds
     a row per token (all of a token's pairs read it), else a row per pair.  gated: N_w = 2 N, out[p] =
-    silu(w[e, :N] a) * (w[e, N:] a); else out[p] = w[e] a, or relu(w[e] a)^2 with activation "relu2".
-    out [pairs, N]: a's dtype, or fp32."""
+    silu(w[e, :N] a) * (w[e, N:] a), or with limit > 0 the gated activation with limits (`clamped_gate`); else
+    out[p] = w[e] a, or relu(w[e] a)^2 with activation "relu2".  out [pairs, N]: a's dtype, or fp32."""
+    if limit < 0 or (limit and not gated):
+        raise KernelError("moe_gemm: a limit (positive) belongs to a gated product")
     _check(a, "a", (F32, BF16), (None, None))
     K = a.shape[1]
     pairs = route.num_tokens * route.top
@@ -1493,7 +1509,7 @@ def moe_gemm(a, w, route: ExpertRoute, out, gated: bool, per_token: bool, activa
         raise KernelError("moe_gemm: the activated product's result has the inputs' dtype")
     call("as_moe_gemm", _ptr(a), _DT[a.dtype], route.top if per_token else 1, _ptr(w), N, K,
          2 if activation else int(bool(gated)),
-         _ptr(route.order), _ptr(route.tiles), _ptr(route.counts), route.max_tiles, _ptr(out), _DT[out.dtype], _stream())  # fmt: skip
+         _ptr(route.order), _ptr(route.tiles), _ptr(route.counts), route.max_tiles, _ptr(out), _DT[out.dtype], float(limit), _stream())  # fmt: skip
 
 
 def moe_combine(pair_out, top: int, weight: float, out, pair_weight=None, add=None) -> None:
@@ -1508,3 +1524,198 @@ def moe_combine(pair_out, top: int, weight: float, out, pair_weight=None, add=No
         _check(add, "add", out.dtype, (T, N))
     call("as_moe_combine", _ptr(pair_out), top, float(weight), N, _ptr(out), _DT[out.dtype], T, _ptr(pair_weight),
          _ptr(add), _stream())  # fmt: skip
+
+
+# ---- what a layer does to the stream around its parts ------------------------------------------------------
+
+NORM_MAX_GROUPS = 256
+CLAMPED_GATE_ALPHA = 1.702  # the factor inside the sigmoid of the gated activation with limits
+
+
+def group_norm(x, weight, eps, groups: int, out, delta=None, rows=None, update_x=True) -> None:
+    """out[r] = the RMS norm in `groups` equal parts of x[s] (+ delta[s]), times weight; s = rows[r] or r.  x fp32
+    [T, n] (receives the sum if update_x), weight fp32 [n], delta and out in the compute dtype."""
+    _check(x, "x", F32, (None, None))
+    T, n = x.shape
+    _check(weight, "weight", F32, (n,))
+    _check(out, "out", (F32, BF16), (None, n))
+    if delta is not None:
+        _check(delta, "delta", out.dtype, (T, n))
+    if rows is not None:
+        _check(rows, "rows", I32, (out.shape[0],))
+    elif out.shape[0] != T:
+        raise KernelError("group_norm: one output row per row of the stream")
+    if not 1 <= groups <= NORM_MAX_GROUPS or n % groups:
+        raise KernelError(f"group_norm: {n} columns do not divide into {groups} groups (at most {NORM_MAX_GROUPS})")
+    call("as_group_norm", _ptr(x), _ptr(delta), _ptr(rows), _ptr(weight), float(eps), groups, _ptr(out), _DT[out.dtype],
+         out.shape[0], n, int(bool(update_x)), _stream())  # fmt: skip
+
+
+def group_norm_shift(x, weight, mu, eps, groups: int, step_rows, state, out, writes=True) -> None:
+    """The grouped norm of every token's row and a token shift after it: out[t] = h_t + (h' - h_t) * mu with h' the
+    normed row of the token before, zeros at a sequence's first token, and for a row's first token what its request's
+    slot in `state` [slots, n] fp32 holds; the slot then receives the row's last normed row (unless `writes` is off)."""
+    _check(x, "x", F32, (None, None))
+    T, n = x.shape
+    _check(weight, "weight", F32, (n,))
+    _check(mu, "mu", F32, (n,))
+    _check(out, "out", (F32, BF16), (T, n))
+    _check(state, "state", F32, (None, n))
+    _check_rows(step_rows, T)
+    tok_row, row_first, row_len, row_start, row_slots = step_rows
+    if not 1 <= groups <= NORM_MAX_GROUPS or n % groups:
+        raise KernelError(f"group_norm_shift: {n} columns do not divide into {groups} groups (at most {NORM_MAX_GROUPS})")
+    call("as_group_norm_shift", _ptr(x), _ptr(weight), _ptr(mu), float(eps), groups, _ptr(tok_row), _ptr(row_first),
+         _ptr(row_len), _ptr(row_start), _ptr(row_slots), _ptr(state), _ptr(out), _DT[out.dtype], T, n,
+         int(bool(writes)), _stream())  # fmt: skip
+
+
+def depth_average(x, delta, kept, coef, n: int) -> None:
+    """v = x + delta is kept as kept[n]; x = sum_(j < n) coef[j] kept[j] + coef[n] v.  x fp32 [T, w]; delta [T, w] in
+    the compute dtype or None; kept fp32 [slots > n, T, w]; coef fp32 [n + 1]."""
+    _check(x, "x", F32, (None, None))
+    _check(kept, "kept", F32, (None, *x.shape))
+    _check(coef, "coef", F32, (n + 1,))
+    if not 0 <= n < kept.shape[0]:
+        raise KernelError(f"depth_average: result {n} of {kept.shape[0]} kept")
+    dtype = F32
+    if delta is not None:
+        _check(delta, "delta", (F32, BF16), tuple(x.shape))
+        dtype = delta.dtype
+    call("as_depth_average", _ptr(x), _ptr(delta), _DT[dtype], _ptr(kept), _ptr(coef), n, x.numel(), _stream())
+
+
+def clamped_gate(gate_up, out, limit: float) -> None:
+    """out = g sigmoid(1.702 g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit); gate_up [T, 2 I]:
+    a row's gate values, then its up values."""
+    _check(gate_up, "gate_up", (F32, BF16), (None, None))
+    T, two_i = gate_up.shape
+    if two_i % 2 or not limit > 0:
+        raise KernelError("clamped_gate: gate and up come in equal numbers, and the limit is positive")
+    _check(out, "out", gate_up.dtype, (T, two_i // 2))
+    call("as_clamped_gate", _ptr(gate_up), _ptr(out), _DT[gate_up.dtype], T, two_i // 2, float(limit), CLAMPED_GATE_ALPHA,
+         _stream())  # fmt: skip
+
+
+def gemm_clamped_gate(a, w, out, limit: float, choices=None) -> None:
+    """out = clamped_gate(a @ w^T, limit): w [2 I, K] holds the gate rows, then the up rows; out [T, I]."""
+    gate_up = torch.empty((a.shape[0], _rows(w).shape[0]), dtype=a.dtype, device=a.device)
+    gemm(a, w, gate_up, choices)
+    clamped_gate(gate_up, out, limit)
+
+
+# ---- linear attention with a fixed decay per head -------------------------------------------------------------
+
+ACTIVATIONS = {None: 0, "silu": 1, "sigmoid": 2}
+DECAY_SCAN_MAX_DIM = 512
+
+
+def decay_scan(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out,
+               writes=True) -> None:  # fmt: skip
+    """S = decay_h S + k v^T, o = S^T q per head and token, in the order of a row's tokens.  q, k [heads, dim] and v
+    [heads, vdim] are columns q_off.., k_off.., v_off.. of proj [T, ld] after `activation` (None or "silu"), k also
+    times k_scale.  decay fp32 [heads]; state fp32 [slots, heads, dim, vdim]; out fp32 [T, heads, vdim]."""
+    _check(proj, "proj", (F32, BF16), (None, None))
+    T, ld = proj.shape
+    H, D, E = num_heads, dim, vdim
+    if activation not in (None, "silu"):
+        raise KernelError(f"decay_scan: activation {activation!r} (None or 'silu')")
+    if min(H, D, E) < 1 or D > DECAY_SCAN_MAX_DIM or max(q_off + H * D, k_off + H * D, v_off + H * E) > ld or min(q_off, k_off, v_off) < 0:
+        raise KernelError(f"decay_scan: {H} heads of {D} and {E} at columns {q_off}, {k_off}, {v_off} of {ld}")
+    _check(decay, "decay", F32, (H,))
+    _check(state, "state", F32, (None, H, D, E))
+    _check(out, "out", F32, (T, H, E))
+    R = _check_rows(step_rows, T)
+    _, row_first, row_len, row_start, row_slots = step_rows
+    call("as_decay_scan", _ptr(proj), _DT[proj.dtype], ld, q_off, k_off, v_off, H, D, E, ACTIVATIONS[activation],
+         float(k_scale), _ptr(decay), _ptr(state), _ptr(row_first), _ptr(row_len), _ptr(row_start), _ptr(row_slots), R,
+         _ptr(out), int(bool(writes)), _stream())  # fmt: skip
+
+
+def decay_attention(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out,
+                    writes=True) -> None:  # fmt: skip
+    """`decay_scan`'s contract, by whichever kernel suits the step."""
+    decay_scan(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out, writes)
+
+
+def decay_finish(o, groups: int, eps, gain, proj, g_off, gate_activation, out) -> None:
+    """out = norm(o) * gain * act(gate): o fp32 [T, n] normed in `groups` equal parts (RMS, eps inside the root),
+    gain fp32 [n] or None, the gate columns g_off.. of proj [T, ld], act "sigmoid" or "silu"; out [T, n] proj's dtype."""
+    _check(o, "o", F32, (None, None))
+    T, n = o.shape
+    _check(proj, "proj", (F32, BF16), (T, None))
+    if gain is not None:
+        _check(gain, "gain", F32, (n,))
+    _check(out, "out", proj.dtype, (T, n))
+    if gate_activation not in ("silu", "sigmoid") or groups < 1 or n % groups or g_off < 0 or g_off + n > proj.shape[1]:
+        raise KernelError(f"decay_finish: {groups} groups of {n}, gate {gate_activation!r} at column {g_off}")
+    call("as_decay_finish", _ptr(o), n, groups, float(eps), _ptr(gain), _ptr(proj), _DT[proj.dtype], proj.shape[1], g_off,
+         ACTIVATIONS[gate_activation], _ptr(out), T, _stream())  # fmt: skip
+
+
+# ---- attention through a latent ---------------------------------------------------------------------------------
+
+
+def rows_rms_norm(proj, off, n, gain, eps, out) -> None:
+    """out = RMS norm of columns off..off + n of proj [T, ld], times gain fp32 [n]; out [T, n] proj's dtype."""
+    _check(proj, "proj", (F32, BF16), (None, None))
+    _check(gain, "gain", F32, (n,))
+    _check(out, "out", proj.dtype, (proj.shape[0], n))
+    if off < 0 or off + n > proj.shape[1]:
+        raise KernelError("rows_rms_norm: columns outside the rows")
+    call("as_rows_rms_norm", _ptr(proj), _DT[proj.dtype], proj.shape[1], off, n, _ptr(gain), float(eps), _ptr(out),
+         proj.shape[0], _stream())  # fmt: skip
+
+
+def latent_kv_store(proj, off, rank, rot, gain, eps, cos_sin, slots, k_pages, v_pages) -> None:
+    """Columns off.. of proj [T, ld]: `rank` of the latent (RMS-normed here, times gain fp32 [rank]) and `rot` of the
+    shared key part (turned here by cos_sin [T, rot/2, 2] fp32).  [latent | key part | zeros] goes to the key pages
+    [pages, 1, bs, width] at slots[t] (< 0: nowhere), [latent | zeros] to the value pages [pages, 1, width, bs]."""
+    _check(proj, "proj", (F32, BF16), (None, None))
+    T, ld = proj.shape
+    _check(gain, "gain", F32, (rank,))
+    _check(slots, "slots", I32, (T,))
+    _check(k_pages, "k_pages", proj.dtype, (None, 1, None, None))
+    pages, _, bs, width = k_pages.shape
+    _check(v_pages, "v_pages", proj.dtype, (pages, 1, width, bs))
+    if rot:
+        _check(cos_sin, "cos_sin", F32, (T, rot // 2, 2))
+    if rank < 1 or rot < 0 or rot % 2 or rank + rot > width or off < 0 or off + rank + rot > ld:
+        raise KernelError(f"latent_kv_store: a latent of {rank} and a key part of {rot} in pages of {width}, rows of {ld}")
+    call("as_latent_kv_store", _ptr(proj), _DT[proj.dtype], ld, off, rank, rot, _ptr(gain), float(eps), _ptr(cos_sin),
+         _ptr(slots), _ptr(k_pages), _ptr(v_pages), bs, width, T, _stream())  # fmt: skip
+
+
+def latent_q_absorb(q, uk, num_heads, dim, rot, rank, cos_sin, out) -> None:
+    """q [T, heads * (dim + rot)], uk [heads * dim, rank]: out[t, h] = [uk_h^T q_h[:dim] | q_h[dim:] turned by
+    cos_sin | zeros]; out [T, heads, width]."""
+    _check(q, "q", (F32, BF16), (None, num_heads * (dim + rot)))
+    T = q.shape[0]
+    _check(uk, "uk", q.dtype, (num_heads * dim, rank))
+    _check(out, "out", q.dtype, (T, num_heads, None))
+    if rot:
+        _check(cos_sin, "cos_sin", F32, (T, rot // 2, 2))
+    if rank + rot > out.shape[2] or rot % 2:
+        raise KernelError("latent_q_absorb: the latent and the turned part exceed the output's width")
+    call("as_latent_q_absorb", _ptr(q), _ptr(uk), _DT[q.dtype], num_heads, dim, rot, rank, _ptr(cos_sin), _ptr(out),
+         out.shape[2], T, _stream())  # fmt: skip
+
+
+def latent_v_expand(heads, uv_t, rank, gate, g_off, out) -> None:
+    """heads [T, H, width] (the first `rank` coordinates count), uv_t [H, rank, E]: out[t, h E + e] = (sum_r heads[t, h,
+    r] uv_t[h, r, e]) * sigmoid(gate[t, g_off + h E + e]); gate [T, ld] or None (no gate); out [T, H * E]."""
+    _check(heads, "heads", (F32, BF16), (None, None, None))
+    T, H, width = heads.shape
+    _check(uv_t, "uv_t", heads.dtype, (H, rank, None))
+    E = uv_t.shape[2]
+    _check(out, "out", heads.dtype, (T, H * E))
+    ld = 0
+    if gate is not None:
+        _check(gate, "gate", heads.dtype, (T, None))
+        ld = gate.shape[1]
+        if g_off < 0 or g_off + H * E > ld:
+            raise KernelError("latent_v_expand: the gate's columns lie outside its rows")
+    if rank > width:
+        raise KernelError("latent_v_expand: the latent is wider than the heads")
+    call("as_latent_v_expand", _ptr(heads), _ptr(uv_t), _DT[heads.dtype], H, E, rank, width, _ptr(gate), ld, g_off,
+         _ptr(out), T, _stream())  # fmt: skip

@@ -112,7 +112,17 @@ class DecoderModel:
             for name in asked(self.blocks[r.layer].parts()["mixer"]):
                 if ident(cid, name) not in requests:
                     raise ValueError(f"run {i} reads cache {cid}, which no run writes")
+        # what a layer keeps beside its mixer belongs to the run, whatever cache the run's mixer reads
+        for i, r in enumerate(self.plan.run):
+            for name, req in (self.blocks[r.layer].cache_request() or {}).items():
+                requests[(self.layer_cache_id(i), name)] = req
         return requests
+
+    @staticmethod
+    def layer_cache_id(run_index: int) -> int:
+        """The id under which run `run_index` files what its layer keeps itself: apart from every mixer's (those
+        are run indices, from 0 up)."""
+        return -1 - run_index
 
     # ---- one pass ---------------------------------------------------------------------
     def row_splits(self) -> tuple:
@@ -142,8 +152,12 @@ class DecoderModel:
             # the norm that the run after this one starts with: this run's last product may add
             # into x and leave that norm pending instead of handing over a delta
             follows = self.blocks[p.run[i + 1].layer].first_norm() if i + 1 < len(p.run) else None
-            delta = self.blocks[r.layer].forward(x, delta, step, step.cache_view(p.cache_id(i), r.writes),
-                                                 next_norm=follows)  # fmt: skip
+            block = self.blocks[r.layer]
+            extra = {}
+            kept = block.cache_request()
+            if kept:
+                extra["own"] = {name: step.cache_view((self.layer_cache_id(i), name), True) for name in kept}
+            delta = block.forward(x, delta, step, step.cache_view(p.cache_id(i), r.writes), next_norm=follows, **extra)
         return self._head(x, delta, step, logits)
 
     def _reenter(self, x, delta, x0):

@@ -232,6 +232,12 @@ class Arrangement:
         """The norm this layer applies to the stream first, for the layer before to leave pending."""
         return None
 
+    def cache_request(self) -> Optional[dict]:
+        """What the layer itself keeps between steps, beside what its mixer keeps: None, or a dict name ->
+        `StateCacheRequest`.  Every run of the layer has these for itself (also a run whose mixer reads another
+        run's cache); `forward` is then handed the views as `own=` {name: view}."""
+        return None
+
     def forward(self, x, delta, step, cache, next_norm=None):
         raise NotImplementedError
 
@@ -259,4 +265,6 @@ def build(family: str, spec: Any, env: BuildEnv):
 
 
 def _load_builtin() -> None:
-    from atomserve_amd.parts import attention, block, experts, mlp, norm, recurrent, rope  # noqa: F401
+    from atomserve_amd.parts import (  # noqa: F401
+        attention, block, experts, latent_attention, linear_attention, mlp, norm, recurrent, rope,
+    )

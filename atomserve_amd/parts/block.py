@@ -3,6 +3,8 @@
 "prenorm":    x += mixer(norm(x));  x += ffn(norm(x))   (reference atomserve/model.py:378-382)
 "two_norms":  x += mixer(norm1(x)) + ffn(norm2(x)), both parts reading the same x through a norm each
 "gated_prenorm": x += m g1(h) * mixer(h), h = norm(x);  x += m g2(h) * ffn(h), h = norm(x), with sigmoid gates g
+"depth_prenorm": "prenorm" whose mixer may read a token-shifted norm, and whose result may be averaged with the
+              results of all layers before it
 
 The residual stream `x` is fp32 in both precisions.  A part's output is not added at
 once: it travels as the pending `delta` to the next norm, whose kernel adds it into
@@ -11,7 +13,20 @@ products around them instead: a part's last product adds into `x` and leaves the
 pending (`Norm.absorb`), and the next part's first product finishes it (`PendingNorm`).
 """
 
-from atomserve_amd.parts.base import Arrangement, DeltaSum, GatedDelta, PendingNorm, build, register
+import torch
+
+from atomserve_amd.kernels import ops
+from atomserve_amd.parts.base import (
+    Arrangement,
+    DeltaSum,
+    GatedDelta,
+    Part,
+    PendingNorm,
+    StateCacheRequest,
+    WeightDecl,
+    build,
+    register,
+)
 
 
 class PreNormBlock(Arrangement):
@@ -132,3 +147,94 @@ class GatedPreNormBlock(Arrangement):
 
 
 register("arrangement", "gated_prenorm", GatedPreNormBlock)
+
+
+class LayerVectors(Part):
+    """The small tensors that a layer owns beside its norms and parts: the token shift's weights [hidden] and the
+    depth average's [depth_index + 2]; fp32 once bound."""
+
+    capturable = True
+
+    def weight_decls(self) -> dict:
+        s, decls = self.spec, {}
+        if s.token_shift:
+            decls["shift"] = WeightDecl((s.mixer_norm.size,), role="vector")
+        if s.depth_slots:
+            decls["depth"] = WeightDecl((s.depth_index + 2,), role="vector")
+        return decls
+
+    def bind(self, tensors: dict) -> None:
+        super().bind({name: t.float().contiguous() for name, t in tensors.items()})
+
+
+class DepthPreNormBlock(Arrangement):
+    """x += mixer(h), h = norm1(x);  x += ffn(norm2(x))  (spec.ffn None: the mixer alone), with two options.
+
+    spec.token_shift: the mixer reads h_t + (h_(t-1) - h_t) * shift instead of h_t, h_(t-1) the normed row of the
+    token before (zeros before a sequence's first token).  A request's last normed row waits in a state slot of the
+    layer's own for the request's next row, so a prompt may be cut anywhere.
+
+    spec.depth_slots: with X_0 what the embedding gave and X_(i+1) this layer's result (i = spec.depth_index), the
+    stream goes on as sum_(j <= i+1) depth[j] X_j.  The X_j of a step are kept in fp32 in the step's shared
+    results; the layer leaves the stream complete (nothing pending), so the next layer's norm adds nothing."""
+
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        self.mixer_norm = build("norm", spec.mixer_norm, env)
+        self.mixer = build("mixer", spec.mixer, env)
+        self.ffn_norm = self.ffn = None
+        if spec.ffn is not None:
+            self.ffn_norm = build("norm", spec.ffn_norm, env)
+            self.ffn = build("feed_forward", spec.ffn, env)
+        self.vectors = LayerVectors(spec, env)
+        if spec.token_shift and not hasattr(self.mixer_norm, "forward_shifted"):
+            raise ValueError(f"a norm of kind {spec.mixer_norm.kind!r} has no kernel with a token shift")
+        if spec.depth_slots and not 0 <= spec.depth_index < spec.depth_slots - 1:
+            raise ValueError(f"layer result {spec.depth_index + 1} does not fit {spec.depth_slots} kept results")
+
+    def parts(self) -> dict:
+        parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        if self.ffn is not None:
+            parts.update(ffn_norm=self.ffn_norm, ffn=self.ffn)
+        if self.vectors.weight_decls():
+            parts["vectors"] = self.vectors
+        return parts
+
+    def cache_request(self):
+        if self.spec.token_shift:
+            return {"shift": StateCacheRequest((self.spec.mixer_norm.size,), torch.float32)}
+        return None
+
+    def first_norm(self):
+        return None  # nothing is left pending inside a product for this layer
+
+    def forward(self, x, delta, step, cache, next_norm=None, own=None):
+        if isinstance(delta, (PendingNorm, DeltaSum, GatedDelta)):
+            raise ValueError("a layer of this arrangement takes a plain pending output, or none")
+        s = self.spec
+        if s.depth_slots and s.depth_index == 0:
+            if delta is not None:
+                raise ValueError("the first of the layers whose results are averaged starts from a complete stream")
+            kept = step.shared["depth_results"] = torch.empty((s.depth_slots, *x.shape), dtype=torch.float32, device=x.device)
+            kept[0].copy_(x)
+        if s.token_shift:
+            if delta is not None:  # the shift's kernel reads neighbouring rows of a complete stream
+                self.mixer_norm.forward(x, delta)
+            kept_rows = own["shift"]
+            rows = (None if step.decode_only else step.tok_row, step.row_first, step.row_len, step.row_start, step.row_slots)
+            h = self.mixer_norm.forward_shifted(x, self.vectors.shift, rows, kept_rows.state, writes=kept_rows.writes)
+        else:
+            h = self.mixer_norm.forward(x, delta)
+        delta = self.mixer.forward(h, step, cache)
+        if self.ffn is not None:
+            delta = self.ffn.forward(self.ffn_norm.forward(x, delta), step)
+        if not s.depth_slots:
+            return delta
+        kept = step.shared.get("depth_results")
+        if kept is None or kept.shape[0] != s.depth_slots or kept.shape[1:] != x.shape:
+            raise ValueError("the layers whose results are averaged run in order, from the first, within one step")
+        ops.depth_average(x, delta, kept, self.vectors.depth, s.depth_index + 1)
+        return None
+
+
+register("arrangement", "depth_prenorm", DepthPreNormBlock)

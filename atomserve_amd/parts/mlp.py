@@ -1,5 +1,6 @@
 """Dense gated feed-forward: down( act(gate(x)) * up(x) ) with gate and up stacked into
-one matrix (reference atomserve/model.py:339-360)."""
+one matrix (reference atomserve/model.py:339-360).  Activation "silu" is that formula; "clamped_swish" is
+g sigmoid(1.702 g) (u + 1) with g = min(gate, limit) and u = clamp(up, -limit, limit)."""
 
 import torch
 
@@ -14,8 +15,10 @@ class GatedMLP(FeedForward):
 
     def __init__(self, spec, env):
         super().__init__(spec, env)
-        if spec.activation != "silu":
-            raise ValueError(f"activation {spec.activation!r} has no kernel (only 'silu')")
+        if spec.activation not in ("silu", "clamped_swish"):
+            raise ValueError(f"activation {spec.activation!r} has no kernel ('silu' or 'clamped_swish')")
+        if spec.activation == "clamped_swish" and not spec.limit > 0:
+            raise ValueError("the activation with limits needs a positive limit")
 
     def weight_decls(self) -> dict:
         s = self.spec
@@ -38,7 +41,9 @@ class GatedMLP(FeedForward):
         pending = isinstance(h, PendingNorm)
         T, device = (h.x.shape[0], h.x.device) if pending else (h.shape[0], h.device)
         act = torch.empty((T, s.intermediate_size), dtype=env.dtype, device=device)
-        if not (pending and h.gemm_gated(self.gate_up, act, s.activation)):
+        if s.activation == "clamped_swish":
+            ops.gemm_clamped_gate(h.rows() if pending else h, self.gate_up, act, s.limit, env.products)
+        elif not (pending and h.gemm_gated(self.gate_up, act, s.activation)):
             ops.gemm_silu_mul(h.rows() if pending else h, self.gate_up, act, env.products)
         if residual is not None and next_norm is not None:
             link = next_norm.absorb(act, self.down, residual)

@@ -93,3 +93,42 @@ class RMSNorm(Norm):
 
 
 register("norm", "rmsnorm", RMSNorm)
+
+
+class GroupedRMSNorm(Norm):
+    """An RMS norm in groups: the row is cut into spec.groups equal consecutive parts, each divided by its own
+    sqrt(mean(part^2) + eps), and the whole multiplied by the gain.  `forward` is the plain norm's (pending residual
+    sum, row selection); `forward_shifted` also mixes every token's normed row with the one of the token before."""
+
+    capturable = True
+
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        if spec.groups < 1 or spec.size % spec.groups or spec.groups > ops.NORM_MAX_GROUPS:
+            raise ValueError(f"a norm of {spec.size} does not divide into {spec.groups} groups (at most {ops.NORM_MAX_GROUPS})")
+
+    def weight_decls(self) -> dict:
+        return {"weight": WeightDecl((self.spec.size,), role="vector")}
+
+    def bind(self, tensors: dict) -> None:
+        super().bind(tensors)
+        self.gain_f32 = self.weight.float().contiguous()  # exact: what a file holds in 16 bits widens
+
+    def forward(self, x, delta=None, rows=None, update_residual=True) -> torch.Tensor:
+        if delta is not None and not isinstance(delta, torch.Tensor):
+            raise ValueError("a grouped norm adds a plain pending output into the stream")
+        n_out = x.shape[0] if rows is None else rows.shape[0]
+        out = torch.empty((n_out, self.spec.size), dtype=self.env.dtype, device=x.device)
+        ops.group_norm(x, self.gain_f32, self.spec.eps, self.spec.groups, out, delta=delta, rows=rows,
+                       update_x=update_residual)  # fmt: skip
+        return out
+
+    def forward_shifted(self, x, mu, step_rows, state, writes=True) -> torch.Tensor:
+        """norm(x) with a token shift by mu (fp32 [size]): out_t = h_t + (h_(t-1) - h_t) * mu.  state fp32 [slots, size]
+        holds every request's last normed row between its rows; step_rows as the kernels of mixers with state take them."""
+        out = torch.empty((x.shape[0], self.spec.size), dtype=self.env.dtype, device=x.device)
+        ops.group_norm_shift(x, self.gain_f32, mu, self.spec.eps, self.spec.groups, step_rows, state, out, writes=writes)
+        return out
+
+
+register("norm", "grouped_rmsnorm", GroupedRMSNorm)

@@ -12,9 +12,13 @@ from typing import Any, Optional
 
 @dataclass(frozen=True)
 class NormSpec:
-    kind: str  # "rmsnorm"
+    """kind "rmsnorm": x / sqrt(mean(x^2) + eps) * gain.  kind "grouped_rmsnorm": the row is cut into `groups` equal
+    consecutive parts, each divided by its own root mean square, the whole times the gain."""
+
+    kind: str
     size: int
     eps: float
+    groups: int = 1
 
 
 @dataclass(frozen=True)
@@ -25,6 +29,67 @@ class RotarySpec:
     kind: str
     rotary_dim: int
     theta: float
+
+
+@dataclass(frozen=True)
+class ScaledRotarySpec:
+    """A rotation ("rope_half" layout) whose frequencies are stretched for contexts beyond `original` positions:
+    with dim(t) = rotary_dim ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(dim(fast)), 0), hi =
+    min(ceil(dim(slow)), rotary_dim - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns by
+    position * (f_i / factor * ramp_i + f_i (1 - ramp_i)), and cosines and sines are multiplied by 0.1 ln(factor) + 1.
+    kind "rope_half_scaled"."""
+
+    kind: str
+    rotary_dim: int
+    theta: float
+    factor: float
+    original: float
+    fast: float
+    slow: float
+
+
+@dataclass(frozen=True)
+class DecayAttentionSpec:
+    """Linear attention with a fixed decay per head and no softmax: S = decay_h S + k v^T, o = S^T q.  q, k
+    [heads, key_dim] and v [heads, value_dim] pass `activation` (None or "silu"); k is also multiplied by `key_scale`.
+    out_norm "heads": every head's o is divided by its root mean square, no gain; "all": the concatenated heads are
+    RMS-normed together and multiplied by a gain.  The result times `gate` ("sigmoid" or "silu") of a projection of
+    the input goes through the output projection."""
+
+    kind: str  # "decay_attention"
+    hidden_size: int
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    decay: tuple  # per head
+    activation: Optional[str]
+    key_scale: float
+    out_norm: str
+    out_norm_eps: float
+    gate: str
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Causal softmax attention whose keys and values are matrices times a cached latent [kv_rank] per token, beside
+    one rotated key part [rot_dim] shared by all heads; queries pass a normed latent of their own [q_rank] and are,
+    per head, `head_dim` coordinates that are not rotated and then `rot_dim` that are.  score = scale (q . k of both
+    parts).  The concatenated heads [heads, value_dim] times sigmoid of a projection of the input go through the
+    output projection.  own_latent False: the layer has no projection to the latent; it reads the pages of the run
+    that its run names as its cache."""
+
+    kind: str  # "latent_attention"
+    hidden_size: int
+    num_heads: int
+    head_dim: int
+    rot_dim: int
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    norm_eps: float
+    position: Any  # of the rot_dim coordinates; a position spec of pairs "half", or None
+    own_latent: bool = True
 
 
 @dataclass(frozen=True)
@@ -71,7 +136,8 @@ class GatedMLPSpec:
     kind: str  # "gated_mlp"
     hidden_size: int
     intermediate_size: int
-    activation: str  # "silu"
+    activation: str  # "silu": silu(gate) * up; "clamped_swish": g sigmoid(1.702 g) (u + 1), g = min(gate, limit), u = clamp(up, +-limit)
+    limit: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -170,13 +236,38 @@ class RoutedExpertsSpec:
 
 
 @dataclass(frozen=True)
+class GatedRoutedExpertsSpec:
+    """Gated experts chosen by a router: z = router h + bias in fp32, the `top` largest z are chosen and weigh the
+    softmax over the chosen z alone (`score` "softmax_of_chosen").  An expert is down(act(gate h, up h)) with the
+    activation of `GatedMLPSpec` and `limit`.  shared_size > 0: one more such expert (with `shared_limit`) runs for
+    every token and is added."""
+
+    kind: str  # "gated_routed_experts"
+    hidden_size: int
+    intermediate_size: int
+    num_experts: int
+    top: int
+    activation: str
+    limit: float
+    score: str = "softmax_of_chosen"
+    router_bias: bool = True
+    shared_size: int = 0
+    shared_limit: float = 0.0
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: a mixer and a feed-forward with their norms, and how they are arranged.
     arrangement "prenorm": x += mixer(norm(x)); x += ffn(norm(x)).
     arrangement "two_norms": x += mixer(mixer_norm(x)) + ffn(ffn_norm(x)), both of the same x
     (ffn and ffn_norm None: the mixer alone).
     arrangement "gated_prenorm": x += m g(h) * mixer(h), h = norm(x); then the same with the feed-forward (or
-    none): m = residual_scale, g the sigmoid gate whose logits the part computes from its input (`out_gate`)."""
+    none): m = residual_scale, g the sigmoid gate whose logits the part computes from its input (`out_gate`).
+    arrangement "depth_prenorm": "prenorm" (ffn None: the mixer alone) with two options.  token_shift: what the mixer
+    reads is h_t + (h_(t-1) - h_t) * shift, h the mixer's norm of the stream (zeros before a sequence's first token;
+    the last h is part of a request's state).  depth_slots > 0: the layer's result is kept as number depth_index + 1
+    of depth_slots results (number 0 is what the embedding gave), and the stream goes on as their weighted sum with
+    depth_index + 2 weights of the layer's own."""
 
     arrangement: str
     mixer: Any
@@ -184,6 +275,9 @@ class BlockSpec:
     ffn: Any
     ffn_norm: Optional[NormSpec]
     residual_scale: float = 1.0
+    token_shift: bool = False
+    depth_index: int = 0
+    depth_slots: int = 0
 
 
 @dataclass(frozen=True)

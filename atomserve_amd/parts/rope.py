@@ -7,6 +7,8 @@ formed and range-reduced in fp64 on the device, so that positions in the tens of
 thousands lose nothing; the rotation that uses them is fp32.
 """
 
+import math
+
 import torch
 
 from atomserve_amd.kernels import ops
@@ -37,3 +39,46 @@ class RotaryHalf(Position):
 
 
 register("position", "rope_half", RotaryHalf)
+
+
+class ScaledRotaryHalf(Position):
+    """The same layout with frequencies stretched for long contexts (`ScaledRotarySpec`): low pair indices (fast
+    turns) keep their frequency, high ones are divided by `factor`, a linear ramp between; cosines and sines are
+    multiplied by 0.1 ln(factor) + 1.  Frequencies are made in fp64 here, angles in fp64 on the device."""
+
+    capturable = True
+    pairs = "half"
+
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        s = spec
+        if s.rotary_dim % 2 or s.rotary_dim <= 0:
+            raise ValueError(f"rotary_dim {s.rotary_dim} must be positive and even")
+        if not (s.theta > 1 and s.factor > 0 and s.original > 0 and s.fast > 0 and s.slow > 0):
+            raise ValueError("a scaled rotation needs theta > 1 and positive factor, original, fast and slow")
+        i = torch.arange(0, s.rotary_dim // 2, dtype=torch.float64)
+        freq = float(s.theta) ** (-2.0 * i / s.rotary_dim)
+
+        def dim_of(turns: float) -> float:
+            return s.rotary_dim * math.log(s.original / (2 * math.pi * turns)) / (2 * math.log(s.theta))
+
+        lo = max(math.floor(dim_of(s.fast)), 0)
+        hi = min(math.ceil(dim_of(s.slow)), s.rotary_dim - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        self.inv_freq = (freq / s.factor * ramp + freq * (1.0 - ramp)).to(env.device)
+        self.magnitude = 0.1 * math.log(s.factor) + 1.0
+
+    def prepare(self, step) -> torch.Tensor:
+        key = ("rope_half_scaled", self.spec)
+        table = step.shared.get(key)
+        if table is None:
+            table = torch.empty((step.num_tokens, self.spec.rotary_dim // 2, 2), dtype=torch.float32,
+                                device=self.env.device)  # fmt: skip
+            ops.rope_table(step.positions, self.inv_freq, table)
+            if self.magnitude != 1.0:
+                table.mul_(self.magnitude)
+            step.shared[key] = table
+        return table
+
+
+register("position", "rope_half_scaled", ScaledRotaryHalf)

@@ -1,7 +1,7 @@
 """Random weights from a configuration and a seed, as a model folder or in memory.
 
 One seeded generator draws every tensor in the order the architecture lists them:
-matrices and biases N(0, std), gains 1 + N(0, gain_std), logarithms of rates N(0, 0.5), mixing matrices I + N(0, 0.2), tables
+matrices and biases N(0, std), gains 1 + N(0, gain_std), logarithms of rates N(0, 0.5), fractions sigmoid(N(0, 1)), depth weights N(0, 0.15) with 1 added to the last, mixing matrices I + N(0, 0.2), tables
 of experts as rows of distinct expert numbers.  Values are drawn in fp32 and rounded
 to the storage dtype, so a bfloat16 folder read back in float32 holds the same numbers.
 """
@@ -30,6 +30,11 @@ def random_checkpoint(arch, config, seed: int, dtype=torch.bfloat16, device="cpu
             t = t.mul_(gain_std).add_(1.0)
         elif role == "log_rate":
             t = t.mul_(0.5)
+        elif role == "fraction":  # between 0 and 1
+            t = torch.sigmoid(t)
+        elif role == "depth_weights":  # mostly the last entry, a share of the others
+            t = t.mul_(0.15)
+            t[-1] += 1.0
         elif role == "near_identity":  # a square matrix that mixes: the identity and a fifth of it in noise
             t = t.mul_(0.2).add_(torch.eye(shape[0], device=device))
         else:
