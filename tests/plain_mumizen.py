@@ -200,3 +200,8 @@ def forward(config, W, tokens, bf16=False, dtype=F, layers_out=None):
         if layers_out is not None:
             layers_out.append(x)
     return linear(W["head"], grouped_rms_norm(x, W["final.norm"], eps, groups), bf16).to(torch.float32)
+
+
+def logits(raw, weights, ids, rounded=False):
+    """The plain model's logits [T, vocab] of one sequence (float64 inside); rounded: with bfloat16 activations."""
+    return forward(raw, weights, list(ids), bf16=rounded)
