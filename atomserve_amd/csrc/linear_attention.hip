@@ -7,6 +7,7 @@
 // slot holds, a later row goes on from what the row before left.  Everything after the products is fp32.
 //
 //   decay_scan    token by token: a lane keeps a slice of one column of the state in registers for all of a row's tokens
+//   decay_chunks  32 tokens at a time as four fp32 products on the matrix cores (keys of up to 128 coordinates)
 //   decay_finish  o normed in groups (per head, or all heads together) with an optional gain, times act(gate)
 #include "common.h"
 
@@ -97,6 +98,147 @@ extern "C" int as_decay_scan(const void* proj, int dtype, int ld, int q_off, int
   else if (dtype == DT_BF16)
     decay_scan_kernel<bf16><<<grid, 64, 0, stream>>>((const bf16*)proj, ld, q_off, k_off, v_off, H, D, E, act, k_scale, decay,
                                                      state, row_first, row_len, row_start, row_slots, out, SL, writes);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// ---- a row's tokens in chunks, on the matrix cores in fp32 ---------------------------------------------------
+// Over a chunk of n <= 32 tokens that starts from the state S (token t counts from 0 within the chunk):
+//
+//   o_t = lam^(t+1) S^T q_t + sum_(j <= t) lam^(t-j) (q_t . k_j) v_j          S' = lam^n S + sum_j lam^(n-1-j) k_j v_j^T
+//
+// which is four products: A = Q K^T (masked and weighed), A V, Q S and K^T V, all of fp32 operands with fp32 sums
+// (v_mfma_f32_32x32x2f32).  grid (column groups of 32, heads, rows), four waves a workgroup.  Wave w keeps rows
+// 32 w .. 32 w + 31 of the state's 32 columns in its accumulator registers from the row's first token to its last,
+// sums A and o over the same 32 key coordinates, and the waves' parts meet in LDS.  An accumulator register i of
+// lane l is element (row 8 (i / 4) + 4 (l / 32) + i % 4, column l % 32); as the second operand of the next product
+// it stands for exactly that row, so the state never leaves its registers.
+#define CHUNK 32
+#define CHUNK_DP 128  // keys are padded with zeros to this width: four waves of 32 coordinates
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <typename T>
+__global__ __launch_bounds__(256) void decay_chunk_kernel(const T* __restrict__ proj, int ld, int q_off, int k_off,
+                                                         int v_off, int H, int D, int E, int act, float k_scale,
+                                                         const float* __restrict__ decay, float* __restrict__ state,
+                                                         const int* __restrict__ row_first,
+                                                         const int* __restrict__ row_len,
+                                                         const int* __restrict__ row_start,
+                                                         const int* __restrict__ row_slots, float* __restrict__ out,
+                                                         int writes) {
+  __shared__ float Qs[CHUNK][CHUNK_DP + 1];
+  __shared__ float Ks[CHUNK][CHUNK_DP + 1];
+  __shared__ float Vs[CHUNK][CHUNK + 1];
+  __shared__ float Part[4][CHUNK][CHUNK + 1];
+  __shared__ float As[CHUNK][CHUNK + 1];
+  __shared__ float pw[CHUNK + 1];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, col = lane & 31, half = lane >> 5;
+  const int e0 = blockIdx.x * CHUNK, h = blockIdx.y, r = blockIdx.z;
+  const int first = row_first[r], len = row_len[r], slot = row_slots[r];
+  const float lam = decay[h];
+  float* kept = slot >= 0 ? state + (((size_t)slot * H + h) * D) * E : nullptr;
+  const bool resume = kept && row_start[r] > 0;
+  const bool e_live = e0 + col < E;
+  if (tid <= CHUNK) pw[tid] = powf(lam, (float)tid);
+  floatx16 S;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int d = 32 * w + 8 * (i / 4) + 4 * half + i % 4;
+    S[i] = (resume && e_live && d < D) ? kept[(size_t)d * E + e0 + col] : 0.f;
+  }
+  for (int c0 = 0; c0 < len; c0 += CHUNK) {
+    const int n = min(CHUNK, len - c0);
+    __syncthreads();  // the chunk before has been read (and pw written)
+    for (int idx = tid; idx < CHUNK * CHUNK_DP; idx += 256) {
+      const int t = idx / CHUNK_DP, d = idx % CHUNK_DP;
+      float qv = 0.f, kv = 0.f;
+      if (t < n && d < D) {
+        const T* row = proj + (size_t)(first + c0 + t) * ld;
+        qv = apply_act(to_f32(row[q_off + h * D + d]), act);
+        kv = apply_act(to_f32(row[k_off + h * D + d]), act) * k_scale;
+      }
+      Qs[t][d] = qv;
+      Ks[t][d] = kv;
+    }
+    for (int idx = tid; idx < CHUNK * CHUNK; idx += 256) {
+      const int t = idx / CHUNK, e = idx % CHUNK;
+      Vs[t][e] = (t < n && e0 + e < E) ? apply_act(to_f32(proj[(size_t)(first + c0 + t) * ld + v_off + h * E + e0 + e]), act) : 0.f;
+    }
+    __syncthreads();
+    // A = Q K^T over this wave's 32 coordinates
+    floatx16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int d = 32 * w + 8 * (i / 4) + 4 * half + i % 4;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Qs[col][d], Ks[col][d], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) Part[w][8 * (i / 4) + 4 * half + i % 4][col] = acc[i];
+    __syncthreads();
+    for (int idx = tid; idx < CHUNK * CHUNK; idx += 256) {
+      const int t = idx / CHUNK, j = idx % CHUNK;
+      const float a = (Part[0][t][j] + Part[1][t][j]) + (Part[2][t][j] + Part[3][t][j]);
+      As[t][j] = j <= t ? a * pw[t - j] : 0.f;
+    }
+    __syncthreads();
+    // o = A V over this wave's 8 tokens, + lam^(t+1) Q S over its 32 coordinates
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int j = 8 * w + 2 * s + half;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(As[col][j], Vs[j][col], acc, 0, 0, 0);
+    }
+    const float grow = pw[col + 1];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int d = 32 * w + 8 * (i / 4) + 4 * half + i % 4;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(Qs[col][d] * grow, S[i], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) Part[w][8 * (i / 4) + 4 * half + i % 4][col] = acc[i];
+    // S = lam^n S + K^T V, key j weighed by lam^(n-1-j)
+    const float shrink = pw[n];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) S[i] *= shrink;
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      const int j = 2 * s + half;
+      const float kw = j < n ? Ks[j][32 * w + col] * pw[n - 1 - j] : 0.f;
+      S = __builtin_amdgcn_mfma_f32_32x32x2f32(kw, Vs[j][col], S, 0, 0, 0);
+    }
+    __syncthreads();
+    for (int idx = tid; idx < CHUNK * CHUNK; idx += 256) {
+      const int t = idx / CHUNK, e = idx % CHUNK;
+      if (t < n && e0 + e < E)
+        out[((size_t)(first + c0 + t) * H + h) * E + e0 + e] = (Part[0][t][e] + Part[1][t][e]) + (Part[2][t][e] + Part[3][t][e]);
+    }
+  }
+  if (kept && writes && e_live) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int d = 32 * w + 8 * (i / 4) + 4 * half + i % 4;
+      if (d < D) kept[(size_t)d * E + e0 + col] = S[i];
+    }
+  }
+}
+
+extern "C" int as_decay_chunks(const void* proj, int dtype, int ld, int q_off, int k_off, int v_off, int H, int D, int E,
+                               int act, float k_scale, const float* decay, float* state, const int* row_first,
+                               const int* row_len, const int* row_start, const int* row_slots, int num_rows, float* out,
+                               int writes, hipStream_t stream) {
+  if (num_rows <= 0) return AS_OK;
+  if (H <= 0 || D <= 0 || E <= 0 || D > CHUNK_DP || act < 0 || act > 2) return AS_BAD_SHAPE;
+  dim3 grid((E + CHUNK - 1) / CHUNK, H, num_rows);
+  if (grid.y > 65535 || grid.z > 65535) return AS_BAD_SHAPE;
+  if (dtype == DT_F32)
+    decay_chunk_kernel<float><<<grid, 256, 0, stream>>>((const float*)proj, ld, q_off, k_off, v_off, H, D, E, act, k_scale, decay,
+                                                        state, row_first, row_len, row_start, row_slots, out, writes);
+  else if (dtype == DT_BF16)
+    decay_chunk_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)proj, ld, q_off, k_off, v_off, H, D, E, act, k_scale, decay,
+                                                       state, row_first, row_len, row_start, row_slots, out, writes);
   else return AS_BAD_DTYPE;
   return launch_status();
 }

@@ -1632,10 +1632,37 @@ def decay_scan(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_sc
          _ptr(out), int(bool(writes)), _stream())  # fmt: skip
 
 
+DECAY_CHUNKS_MAX_DIM = 128
+
+
+def decay_chunks(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out,
+                 writes=True) -> None:  # fmt: skip
+    """`decay_scan`'s contract, a row's tokens 32 at a time as fp32 products on the matrix cores: with S the state
+    before a chunk of n tokens, o_t = decay^(t+1) S^T q_t + sum_(j <= t) decay^(t-j) (q_t . k_j) v_j and the state
+    after it decay^n S + sum_j decay^(n-1-j) k_j v_j^T.  Keys of up to DECAY_CHUNKS_MAX_DIM coordinates."""
+    _check(proj, "proj", (F32, BF16), (None, None))
+    T, ld = proj.shape
+    H, D, E = num_heads, dim, vdim
+    if activation not in (None, "silu"):
+        raise KernelError(f"decay_chunks: activation {activation!r} (None or 'silu')")
+    if min(H, D, E) < 1 or D > DECAY_CHUNKS_MAX_DIM or max(q_off + H * D, k_off + H * D, v_off + H * E) > ld or min(q_off, k_off, v_off) < 0:
+        raise KernelError(f"decay_chunks: {H} heads of {D} and {E} at columns {q_off}, {k_off}, {v_off} of {ld}")
+    _check(decay, "decay", F32, (H,))
+    _check(state, "state", F32, (None, H, D, E))
+    _check(out, "out", F32, (T, H, E))
+    R = _check_rows(step_rows, T)
+    _, row_first, row_len, row_start, row_slots = step_rows
+    call("as_decay_chunks", _ptr(proj), _DT[proj.dtype], ld, q_off, k_off, v_off, H, D, E, ACTIVATIONS[activation],
+         float(k_scale), _ptr(decay), _ptr(state), _ptr(row_first), _ptr(row_len), _ptr(row_start), _ptr(row_slots), R,
+         _ptr(out), int(bool(writes)), _stream())  # fmt: skip
+
+
 def decay_attention(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out,
                     writes=True) -> None:  # fmt: skip
-    """`decay_scan`'s contract, by whichever kernel suits the step."""
-    decay_scan(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out, writes)
+    """`decay_scan`'s contract, by whichever kernel suits the step: token by token where every row is one token (a
+    decode step: step_rows names no row per token) or the keys are wider than the chunked kernel takes, else in chunks."""
+    kernel = decay_scan if step_rows[0] is None or dim > DECAY_CHUNKS_MAX_DIM else decay_chunks
+    kernel(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out, writes)
 
 
 def decay_finish(o, groups: int, eps, gain, proj, g_off, gate_activation, out) -> None:

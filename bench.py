@@ -4,6 +4,7 @@
     python bench.py --workload mixed --sizes 0.6b      (a continuous batch through the scheduler)
     python bench.py --design dozusun [--widths 1024,2048,4096]   (Dozusun layers beside Qwen3 layers of equal size)
     python bench.py --design koravik [--widths 1024,2048,4096]   (Koravik layers beside Qwen3 layers of equal size)
+    python bench.py --design mumizen [--widths 1024,2048,4096]   (Mumizen layers beside Qwen3 layers of equal size)
 
 A step is one decode step of the engine (scheduler, one pass over the GPU, sampling).
 Prints ONE JSON line: decoded tokens per second at batch 8 with 2,048-token contexts,
@@ -76,13 +77,15 @@ def parse_args():
                         "(half of them share their first 32), chunks of 512, 128 tokens decoded each, through the "
                         "scheduler from submission to the last token")  # fmt: skip
     p.add_argument("--chunk-budget", type=int, default=512, help="token budget of a step in the mixed workload")
-    p.add_argument("--design", choices=["qwen3", "dozusun", "koravik"], default="qwen3",
+    p.add_argument("--design", choices=["qwen3", "dozusun", "koravik", "mumizen"], default="qwen3",
                    help="dozusun: prefill and decode throughput of random-weight Dozusun layers (an attention beside a "
                         "gated linear recurrence, gated delta rules, dense and table-routed feed-forwards) at a few "
                         "widths, beside Qwen3 layers of the same width, heads, depth and vocabulary; koravik: the same "
                         "for Koravik layers (attention with mixed heads and kept first tokens, routed experts with a "
-                        "shared one, gated residual sums, a stretch of layers run twice)")  # fmt: skip
-    p.add_argument("--widths", default="1024,2048,4096", help="stream widths of --design dozusun / koravik")
+                        "shared one, gated residual sums, a stretch of layers run twice); mumizen: the same for Mumizen "
+                        "layers (linear attentions with fixed decays, attention through a cached latent, gated "
+                        "feed-forwards with limits, dense and routed, an average over all layers' results)")  # fmt: skip
+    p.add_argument("--widths", default="1024,2048,4096", help="stream widths of --design dozusun / koravik / mumizen")
     p.add_argument("--profile", action="store_true",
                    help="also split the host's time of a decode step into schedule / pack / launch / sample / wait / "
                         "update (steps run one at a time meanwhile, none sent ahead), as the reference's "
@@ -202,12 +205,43 @@ def koravik_config(width: int, layers: int, vocab: int):
                                     "loop": {"start": 1, "stop": 3, "times": 2}})  # fmt: skip
 
 
+def mumizen_config(width: int, layers: int, vocab: int):
+    """Layers as a model of this design of that width would have them: heads of 128 everywhere; the two linear
+    attentions with keys and values of 128 and decays 1 - 2^-(5 + 5 h / heads); attention through a latent of 192
+    beside a turned part of 64 (queries through a latent of half the width, values of 128), every second one reading
+    the latent of the one before; feed-forwards three times the width, dense or as 16 experts of a quarter of that (two
+    to a token) beside a shared expert of one and a half times the width; the four kinds of layers in turn."""
+    from atomserve_amd.config.model_config import MumizenConfig
+
+    heads = width // 128
+    decay = {"heads": heads, "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** -(5.0 + 5.0 * h / heads) for h in range(heads)]}
+    rot = {"dims": 64, "base": 1e6, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    latent = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": width // 2, "kv_rank": 192,
+              "scale": 192**-0.5, "rot": rot}  # fmt: skip
+    dense = {"kind": "dense", "ff": 3 * width, "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": 3 * width // 4, "limit": 7.0}, "router": {"experts": 16, "top": 2},
+           "shared": {"ff": 3 * width // 2, "limit": 7.0}}  # fmt: skip
+    made = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 0:
+            made.append({"type": "lightning", "mixer": decay, "mlp": dense})
+        elif kind == 1:
+            made.append({"type": "latent_attention", "mixer": latent, "mlp": moe})
+        elif kind == 2:
+            made.append({"type": "retention", "mixer": decay, "mlp": dense})
+        else:
+            made.append({"type": "latent_attention", "mixer": dict(latent, kv_from=i - 2), "mlp": moe})
+    return MumizenConfig.from_dict({"architecture": "Mumizen", "vocab": vocab, "width": width,
+                                    "norm": {"eps": 1e-6, "groups": 4}, "layers": made})  # fmt: skip
+
+
 def design_comparison(args) -> dict:
     """Prefill of --prefill-tokens tokens and decode at batch 1 and --batch with --context tokens of context, for
     the layers of --design and for Qwen3 layers of equal width, heads, depth and vocabulary; random weights, the
     engine's own entry point (scheduler, captured decode steps, sampling)."""
     design = args.design
-    make = {"dozusun": dozusun_config, "koravik": koravik_config}[design]
+    make = {"dozusun": dozusun_config, "koravik": koravik_config, "mumizen": mumizen_config}[design]
     import torch
 
     from atomserve_amd.config import EngineConfig, Qwen3Config
@@ -328,7 +362,7 @@ def main() -> int:
     from atomserve_amd.weights.loader import DictSource, bind_checkpoint
     from atomserve_amd.weights.random_init import random_checkpoint
 
-    if args.design in ("dozusun", "koravik"):
+    if args.design in ("dozusun", "koravik", "mumizen"):
         print(json.dumps(design_comparison(args)))
         return 0
     device = "cuda:0"

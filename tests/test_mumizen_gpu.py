@@ -383,8 +383,9 @@ def test_average_over_the_layers_results(dtype):
     assert (y.cpu() - (0.25 * results[0] - 2.0 * results[1])).abs().max() <= 1e-5
 
 
-def run_decay(q, k, v, decay, act, k_scale, cuts, dtype, slot=1, state=None):
-    """The scan over one request cut into rows of `cuts` tokens (one call each), q, k, v given before the activation."""
+def run_decay(q, k, v, decay, act, k_scale, cuts, dtype, slot=1, state=None, kernel=None):
+    """The scan over one request cut into rows of `cuts` tokens (one call each), q, k, v given before the activation.
+    kernel: "decay_scan" or "decay_chunks" to name one; None: as a step would choose (single tokens as a decode step)."""
     from atomserve_amd.kernels import ops
 
     T, H, D = q.shape
@@ -396,8 +397,11 @@ def run_decay(q, k, v, decay, act, k_scale, cuts, dtype, slot=1, state=None):
     outs = []
     for at, n in in_pieces(T, cuts):
         o = torch.empty((n, H, E), dtype=torch.float32, device=DEV)
-        ops.decay_attention(proj[at : at + n].contiguous(), q_off, k_off, v_off, H, D, E, act, k_scale, dev(torch.tensor(decay)),
-                            state, step_rows([n], [at], [slot]), o)  # fmt: skip
+        rows = step_rows([n], [at], [slot])
+        if kernel is None and n == 1:
+            rows = (None, *rows[1:])
+        getattr(ops, kernel or "decay_attention")(proj[at : at + n].contiguous(), q_off, k_off, v_off, H, D, E, act, k_scale,
+                                                  dev(torch.tensor(decay)), state, rows, o)  # fmt: skip
         outs.append(o.cpu())
     return torch.cat(outs), state
 
@@ -418,9 +422,10 @@ def test_linear_attention_with_decays(shape, dtype):
         f = (lambda t: silu(t.double())) if act else (lambda t: t.double())
         want = plain.decayed_state_scan(f(q), f(k) * k_scale, f(v), decay).float()
         tol = 2e-5 * float(want.abs().max())
-        for cuts in ([T], [1] * T, [2, 31, 1, 1, 30, 2]):
-            got, state = run_decay(q, k, v, decay, act, k_scale, cuts, dtype)
-            assert (got - want).abs().max() <= tol, f"{shape} {act} {cuts}: {float((got - want).abs().max()):.3e} of {float(want.abs().max()):.3e}"
+        kernels = ("decay_scan", "decay_chunks") if D <= 128 else ("decay_scan",)
+        for cuts, kernel in [(c, kn) for c in ([T], [1] * T, [2, 31, 1, 1, 30, 2], [32, 33, 2]) for kn in kernels] + [([1] * T, None), ([T], None)]:
+            got, state = run_decay(q, k, v, decay, act, k_scale, cuts, dtype, kernel=kernel)
+            assert (got - want).abs().max() <= tol, f"{shape} {act} {cuts} {kernel}: {float((got - want).abs().max()):.3e} of {float(want.abs().max()):.3e}"
         assert bool((state[0] == 5.0).all()) and bool((state[2] == 5.0).all())  # the other slots are not touched
 
 
@@ -433,13 +438,14 @@ def test_linear_attention_keeps_a_far_key_and_forgets_by_its_decay():
     k, v = torch.zeros(T, H, D), bf(torch.randn(T, H, E, generator=gen))
     k[special] = bf(torch.randn(H, D, generator=gen))
     decay = [1.0, 0.96875]
-    for cuts in ([T], [special, T - special], [special + 1, T - special - 1], [special, 1, 1, 2, T - special - 4], [64] * 6 + [36]):
-        got, _ = run_decay(q, k, v, decay, None, 1.0, cuts, "float32")
+    ways = ([T], [special, T - special], [special + 1, T - special - 1], [special, 1, 1, 2, T - special - 4], [64] * 6 + [36])
+    for cuts, kernel in [(c, kn) for c in ways for kn in ("decay_scan", "decay_chunks")]:
+        got, _ = run_decay(q, k, v, decay, None, 1.0, cuts, "float32", kernel=kernel)
         assert bool((got[:special] == 0).all())
         for t in (special, special + 1, special + 64, T - 1):
             for h in range(H):
                 want = decay[h] ** (t - special) * float(q[t, h] @ k[special, h]) * v[special, h]
-                assert (got[t, h] - want).abs().max() <= 1e-5 * max(1.0, float(want.abs().max())), (cuts, t, h)
+                assert (got[t, h] - want).abs().max() <= 1e-5 * max(1.0, float(want.abs().max())), (cuts, kernel, t, h)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
