@@ -366,7 +366,9 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const int* __restrict__ items, const int* __restrict__ positions, const int* __restrict__ tok_row,
     const int* __restrict__ block_tables, int table_width, bf16* __restrict__ out, float* __restrict__ part_m,
     float* __restrict__ part_l, float* __restrict__ part_acc, int H, int KV, int bs, float scale, int window,
-    int part_size, int P, int cus, FreshQKV fresh) {
+    int part_size, int P, int cus, int share, FreshQKV fresh) {
+  // share > 1: every `share` consecutive kv heads named here are one head of the pages (a group of more query heads
+  // than a workgroup takes, cut into several); the pages then hold KV / share heads.
   constexpr int D = DC * 32, DT = DC * 2;  // DT: tiles of 16 output coordinates
   extern __shared__ float smem[];          // [4][16] m, [4][16] l, [4][D][G] acc
   __shared__ __align__(16) bf16 fresh_kv[2][256];  // FRESH: the new token's key and value
@@ -393,6 +395,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   const int lo = window > 0 ? max(0, ctx - window) : 0;
   const int k0 = max(lo, part * part_size), k1 = min(ctx, (part + 1) * part_size);
   const int h0 = kvh * G;
+  const int page_heads = KV / share, page_head = kvh / share;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;  // col: head within the group (and key row of A)
 
@@ -462,7 +465,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   const int first = (k0 / 32) * 32;
   KVStep<DC> cur, nxt;
   int kb = first + 32 * wave;
-  if (kb < k1) load_kv_step<DC>(cur, k_pages, v_pages, table, kb, k1, KV, kvh, bs, col, grp);
+  if (kb < k1) load_kv_step<DC>(cur, k_pages, v_pages, table, kb, k1, page_heads, page_head, bs, col, grp);
 
   if constexpr (FRESH != 0) {
     // the queries of this lane's head: norm over the head (its D values lie in four lanes), rotation
@@ -533,7 +536,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 
   for (; kb < k1; kb += 128) {
     const bool more = kb + 128 < k1;
-    if (more) load_kv_step<DC>(nxt, k_pages, v_pages, table, kb + 128, k1, KV, kvh, bs, col, grp);
+    if (more) load_kv_step<DC>(nxt, k_pages, v_pages, table, kb + 128, k1, page_heads, page_head, bs, col, grp);
     if constexpr (FRESH != 0) {
       if (fresh_here && pos >= kb && pos < kb + 32) {  // this wave's step holds the token itself: take it from LDS
         const int at = pos - kb;  // = KEY_OF_ROW(tile, row) for
@@ -1134,10 +1137,11 @@ static int launch_decode_mfma(const void* q, const void* k_pages, const void* v_
                               int num_items, const int* positions, const int* tok_row, const int* block_tables,
                               int table_width, void* out, float* part_m, float* part_l, float* part_acc, int H,
                               int KV, int D, int bs, float scale, int window, int part_size, int P,
-                              const FreshQKV* fresh, int gains_dtype, hipStream_t stream) {
+                              const FreshQKV* fresh, int gains_dtype, hipStream_t stream, int share = 1) {
   const int G = H / KV;
   if (D % 32 || D > 256 || G > 16 || bs % 16 || part_size % 32) return AS_BAD_SHAPE;
   if (fresh && D % 64) return AS_BAD_SHAPE;
+  if (share < 1 || KV % share || (fresh && share != 1)) return AS_BAD_SHAPE;
   dim3 grid(num_items, KV, P);
   const size_t shmem = sizeof(float) * (size_t)(128 + 4 * D * G);
   if (shmem + 1024 > (64u << 10)) return AS_BAD_SHAPE;  // wide heads in large groups: the general kernel's
@@ -1146,7 +1150,7 @@ static int launch_decode_mfma(const void* q, const void* k_pages, const void* v_
   attn_decode_mfma_kernel<DCV, FRESHV><<<grid, 256, shmem, stream>>>(                                     \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, items, positions, tok_row, block_tables, \
       table_width, (bf16*)out, part_m, part_l, part_acc, H, KV, bs, scale, window, part_size, P,          \
-      compute_units(), FRESHV ? *fresh : none)
+      compute_units(), share, FRESHV ? *fresh : none)
 #define LAUNCH_FRESH(FRESHV)            \
   switch (D / 64) {                     \
     case 1: LAUNCH(2, FRESHV); break;   \
@@ -1193,6 +1197,22 @@ extern "C" int as_attn_decode_mfma(const void* q, const void* k_pages, const voi
   return launch_decode_mfma(q, k_pages, v_pages, items, num_items, positions, tok_row, block_tables, table_width,
                             out, part_m, part_l, part_acc, H, KV, D, bs, scale, window, part_size, P, nullptr,
                             DT_BF16, stream);
+}
+
+// The same where the pages hold KV / share heads and every `share` consecutive groups of H / KV query heads read
+// one of them: a group of more than 16 query heads, cut into several of equal size.
+extern "C" int as_attn_decode_mfma_shared(const void* q, const void* k_pages, const void* v_pages, const int* items,
+                                          int num_items, const int* positions, const int* tok_row,
+                                          const int* block_tables, int table_width, void* out, float* part_m,
+                                          float* part_l, float* part_acc, int H, int KV, int D, int bs, float scale,
+                                          int window, int part_size, int P, int share, hipStream_t stream) {
+  if (num_items <= 0) return AS_OK;
+  if (H <= 0 || KV <= 0 || H % KV || D <= 0 || bs <= 0 || part_size <= 0 || P <= 0 || table_width <= 0)
+    return AS_BAD_SHAPE;
+  if (P > 1 && (!part_m || !part_l || !part_acc)) return AS_BAD_SHAPE;
+  return launch_decode_mfma(q, k_pages, v_pages, items, num_items, positions, tok_row, block_tables, table_width,
+                            out, part_m, part_l, part_acc, H, KV, D, bs, scale, window, part_size, P, nullptr,
+                            DT_BF16, stream, share);
 }
 
 // A decode step (token t is row t of the block tables) from the projection's output: per-head norm,

@@ -207,8 +207,9 @@ SINGLE_QUERY_MAX_HEAD_DIM = 256
 def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tables, out, scale, window,
                       max_context, part_size=None, force_generic=False) -> None:  # fmt: skip
     """Attention of single query tokens over the paged cache.  bfloat16 with head widths in steps
-    of 32, groups of up to 16 heads and pages of a multiple of 16 tokens runs on the matrix cores;
-    everything else (and all of fp32) on the general kernel.
+    of 32 and pages of a multiple of 16 tokens runs on the matrix cores (a group of more than 16 query
+    heads, or of wide heads that overfill a workgroup's LDS, as several equal groups that read the same kv
+    head); everything else (and all of fp32) on the general kernel.
 
     q, out [T, H, D]; items [N] int32: the tokens (rows of q) to process, None for all of them in
     order; positions, tok_row [T] int32 (tok_row None: token t belongs to row t, a decode step);
@@ -237,8 +238,15 @@ def attn_single_query(q, k_pages, v_pages, items, positions, tok_row, block_tabl
     if max_context > block_tables.shape[1] * bs:
         raise KernelError("attention: block tables are shorter than the longest context")
     G = H // KV
-    mfma = (q.dtype == BF16 and D % 32 == 0 and G <= 16 and bs % 16 == 0 and _decode_mfma_fits(D, G)
-            and not force_generic)  # fmt: skip
+    # a group of more query heads than the matrix-core kernel's workgroup takes is cut into equal smaller ones
+    share = next((G // g for g in range(min(G, 16), 0, -1) if G % g == 0 and _decode_mfma_fits(D, g)), 0)
+    mfma = q.dtype == BF16 and D % 32 == 0 and bs % 16 == 0 and share > 0 and not force_generic
+    if mfma and share > 1:
+        part_size, P, part_m, part_l, part_acc = _partitions(N, H, KV * share, D, max_context, window, True, part_size, q.device)
+        call("as_attn_decode_mfma_shared", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(items), N, _ptr(positions),
+             _ptr(tok_row), _ptr(block_tables), block_tables.shape[1], _ptr(out), _ptr(part_m), _ptr(part_l),
+             _ptr(part_acc), H, KV * share, D, bs, float(scale), int(window), part_size, P, share, _stream())  # fmt: skip
+        return
     part_size, P, part_m, part_l, part_acc = _partitions(N, H, KV, D, max_context, window, mfma, part_size, q.device)
     if mfma:
         call("as_attn_decode_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(items), N, _ptr(positions),
@@ -1637,7 +1645,7 @@ DECAY_CHUNKS_MAX_DIM = 128
 
 def decay_chunks(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out,
                  writes=True) -> None:  # fmt: skip
-    """`decay_scan`'s contract, a row's tokens 32 at a time as fp32 products on the matrix cores: with S the state
+    """What `decay_scan` computes, a row's tokens 32 at a time as fp32 products on the matrix cores: with S the state
     before a chunk of n tokens, o_t = decay^(t+1) S^T q_t + sum_(j <= t) decay^(t-j) (q_t . k_j) v_j and the state
     after it decay^n S + sum_j decay^(n-1-j) k_j v_j^T.  Keys of up to DECAY_CHUNKS_MAX_DIM coordinates."""
     _check(proj, "proj", (F32, BF16), (None, None))
@@ -1659,7 +1667,7 @@ def decay_chunks(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_
 
 def decay_attention(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out,
                     writes=True) -> None:  # fmt: skip
-    """`decay_scan`'s contract, by whichever kernel suits the step: token by token where every row is one token (a
+    """What `decay_scan` computes, by whichever kernel suits the step: token by token where every row is one token (a
     decode step: step_rows names no row per token) or the keys are wider than the chunked kernel takes, else in chunks."""
     kernel = decay_scan if step_rows[0] is None or dim > DECAY_CHUNKS_MAX_DIM else decay_chunks
     kernel(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out, writes)

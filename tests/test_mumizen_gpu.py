@@ -552,7 +552,8 @@ def plain_latent_attention(q, c, kr, uk, uv, scale):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", [(3, 8, 8, 16, 40), (18, 4, 4, 8, 24), (4, 32, 32, 32, 128), (2, 40, 0, 16, 64), (6, 16, 2, 8, 222)])
+@pytest.mark.parametrize("shape", [(3, 8, 8, 16, 40), (18, 4, 4, 8, 24), (4, 32, 32, 32, 128), (2, 40, 0, 16, 64), (6, 16, 2, 8, 222),
+                                   (32, 24, 64, 16, 192), (48, 8, 16, 8, 80)])
 def test_attention_through_a_latent(shape, dtype):
     """Random queries, latents and key parts: heads' keys and values written out from the latent in the plain form,
     absorbed into the queries and applied after the attention in the kernels; as single tokens and in tiles."""
