@@ -11,6 +11,7 @@
 //   latent_kv_store   norm of c, rotation of k_r, [c | k_r] into the key pages and c into the value pages
 //   latent_q_absorb   q [T, H, D + R] -> [U_h^T q_h | rotate(q_h[D:])], zeros up to the pages' width
 //   latent_v_expand   heads [T, H, width] (their first kv_rank coordinates) -> V_h heads, times sigmoid(gate)
+//   wide_attend       the attention itself for latents wider than the paged attention kernels' heads
 //
 // Norms, the rotation and every sum are fp32; an output is one chain of multiply-adds in a fixed order.
 #include "common.h"
@@ -199,6 +200,93 @@ extern "C" int as_latent_v_expand(const void* heads, const void* uv_t, int dtype
     latent_v_expand_kernel<float><<<grid, 256, lds, stream>>>((const float*)heads, (const float*)uv_t, H, E, rank, width, (const float*)gate, ld, g_off, (float*)out, num_tokens);
   else if (dtype == DT_BF16)
     latent_v_expand_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)heads, (const bf16*)uv_t, H, E, rank, width, (const bf16*)gate, ld, g_off, (bf16*)out, num_tokens);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// ---- attention over one kv head of any width ------------------------------------------------------------------
+// For pages whose one head is wider than the paged attention kernels take.  q, out [T, H, width]; k_pages
+// [pages, 1, bs, width], v_pages [pages, 1, width, bs]; a token at position p of row r sees keys 0 .. p of the row's
+// block table.  grid (tokens, heads), 256 threads: the keys come 256 at a time from position 0 (a thread a key, its
+// score one chain of multiply-adds), the softmax's maximum and sum move on from block to block, and a thread owns
+// every 256th coordinate of the output.  All sums are fp32 and taken in an order that only positions decide.
+#define WIDE_MAX_COLS 8  // coordinates of the output a thread owns: widths up to 2,048
+
+template <typename T>
+__global__ __launch_bounds__(256) void wide_attend_kernel(const T* __restrict__ q, const T* __restrict__ k_pages,
+                                                          const T* __restrict__ v_pages,
+                                                          const int* __restrict__ positions,
+                                                          const int* __restrict__ tok_row,
+                                                          const int* __restrict__ block_tables, int table_width,
+                                                          T* __restrict__ out, int H, int width, int bs, float scale) {
+  extern __shared__ float lds[];  // [width] the query, [256] the block's weights
+  __shared__ float red[17];
+  float* qs = lds;
+  float* ps = lds + width;
+  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int ctx = positions[t] + 1;
+  const int* table = block_tables + (size_t)(tok_row ? tok_row[t] : t) * table_width;
+  for (int i = tid; i < width; i += 256) qs[i] = to_f32(q[((size_t)t * H + h) * width + i]) * scale;
+  float acc[WIDE_MAX_COLS];
+#pragma unroll
+  for (int c = 0; c < WIDE_MAX_COLS; ++c) acc[c] = 0.f;
+  float m = -__builtin_inff(), l = 0.f;
+  __syncthreads();
+  for (int k0 = 0; k0 < ctx; k0 += 256) {
+    const int j = k0 + tid;
+    float sc = -__builtin_inff();
+    if (j < ctx) {
+      const T* key = k_pages + ((size_t)table[j / bs] * bs + j % bs) * width;
+      sc = 0.f;
+      for (int i = 0; i < width; ++i) sc = fmaf(qs[i], to_f32(key[i]), sc);
+    }
+    float top = sc;
+    for (int off = 32; off > 0; off >>= 1) top = fmaxf(top, __shfl_xor(top, off, WAVE));
+    if ((tid & 63) == 0) red[tid >> 6] = top;
+    __syncthreads();
+    const float mn = fmaxf(m, fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
+    __syncthreads();
+    const float p = j < ctx ? expf(sc - mn) : 0.f;
+    const float a = expf(m - mn);  // m = -inf in the first block: 0
+    ps[tid] = p;
+    const float sum = block_sum(p, red);  // synchronises: ps is written
+    l = l * a + sum;
+    m = mn;
+    const int here = min(256, ctx - k0);
+#pragma unroll
+    for (int c = 0; c < WIDE_MAX_COLS; ++c) {
+      const int d = tid + 256 * c;
+      if (d < width) {
+        float s = 0.f;
+        for (int jj = 0; jj < here; ++jj) {
+          const int key = k0 + jj;
+          s = fmaf(ps[jj], to_f32(v_pages[((size_t)table[key / bs] * width + d) * bs + key % bs]), s);
+        }
+        acc[c] = acc[c] * a + s;
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int c = 0; c < WIDE_MAX_COLS; ++c) {
+    const int d = tid + 256 * c;
+    if (d < width) out[((size_t)t * H + h) * width + d] = from_f32<T>(acc[c] / l);
+  }
+}
+
+extern "C" int as_wide_attend(const void* q, const void* k_pages, const void* v_pages, int dtype, const int* positions,
+                              const int* tok_row, const int* block_tables, int table_width, void* out, int H, int width,
+                              int bs, float scale, int num_tokens, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (H <= 0 || H > 65535 || width <= 0 || width > 256 * WIDE_MAX_COLS || bs <= 0 || table_width <= 0) return AS_BAD_SHAPE;
+  dim3 grid(num_tokens, H);
+  const size_t lds = (size_t)(width + 256) * sizeof(float);
+  if (dtype == DT_F32)
+    wide_attend_kernel<float><<<grid, 256, lds, stream>>>((const float*)q, (const float*)k_pages, (const float*)v_pages, positions,
+                                                         tok_row, block_tables, table_width, (float*)out, H, width, bs, scale);
+  else if (dtype == DT_BF16)
+    wide_attend_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, positions,
+                                                        tok_row, block_tables, table_width, (bf16*)out, H, width, bs, scale);
   else return AS_BAD_DTYPE;
   return launch_status();
 }

@@ -50,6 +50,7 @@ SIGNATURES = {
     "as_latent_kv_store": ("latent", [P, I, I, I, I, I, P, F, P, P, P, P, I, I, I, P]),
     "as_latent_q_absorb": ("latent", [P, P, I, I, I, I, I, P, P, I, I, P]),
     "as_latent_v_expand": ("latent", [P, P, I, I, I, I, I, P, I, I, P, I, P]),
+    "as_wide_attend": ("latent", [P, P, P, I, P, P, P, I, P, I, I, I, F, I, P]),
     "as_attn_headmix_mfma": ("attention_mix", [P, P, P, P, I, I, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, P, P, P]),
     "as_attn_headmix": ("attention_mix", [P, P, P, I, P, I, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P]),
     "as_attn_single_query": ("attention", [P, P, P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, P]),

@@ -1691,6 +1691,9 @@ def decay_finish(o, groups: int, eps, gain, proj, g_off, gate_activation, out) -
 # ---- attention through a latent ---------------------------------------------------------------------------------
 
 
+LATENT_MAX_RANK, LATENT_MAX_HEAD_DIM = 1536, 1024  # what eight tokens' latents, or heads, may fill of a workgroup's LDS
+
+
 def rows_rms_norm(proj, off, n, gain, eps, out) -> None:
     """out = RMS norm of columns off..off + n of proj [T, ld], times gain fp32 [n]; out [T, n] proj's dtype."""
     _check(proj, "proj", (F32, BF16), (None, None))
@@ -1754,3 +1757,30 @@ def latent_v_expand(heads, uv_t, rank, gate, g_off, out) -> None:
         raise KernelError("latent_v_expand: the latent is wider than the heads")
     call("as_latent_v_expand", _ptr(heads), _ptr(uv_t), _DT[heads.dtype], H, E, rank, width, _ptr(gate), ld, g_off,
          _ptr(out), T, _stream())  # fmt: skip
+
+
+WIDE_ATTEND_MAX_WIDTH = 2048
+
+
+def wide_attend(q, k_pages, v_pages, positions, tok_row, block_tables, out, scale, max_context) -> None:
+    """Causal attention of every token's heads q [T, H, width] over ONE kv head of any width up to
+    WIDE_ATTEND_MAX_WIDTH (k_pages [pages, 1, bs, width], v_pages [pages, 1, width, bs]): for pages wider than the
+    paged attention kernels' heads.  positions, tok_row [T] int32 (tok_row None: token t is row t); out like q."""
+    _check(q, "q", (F32, BF16), (None, None, None))
+    T, H, width = q.shape
+    _check(out, "out", q.dtype, (T, H, width))
+    _check(k_pages, "k_pages", q.dtype, (None, 1, None, width))
+    pages, _, bs, _ = k_pages.shape
+    _check(v_pages, "v_pages", q.dtype, (pages, 1, width, bs))
+    _check(positions, "positions", I32, (T,))
+    if tok_row is not None:
+        _check(tok_row, "tok_row", I32, (T,))
+    _check(block_tables, "block_tables", I32, (None, None))
+    if tok_row is None and block_tables.shape[0] < T:
+        raise KernelError(f"attention: {T} tokens that are their own rows need as many block tables")
+    if width > WIDE_ATTEND_MAX_WIDTH:
+        raise KernelError(f"attention: heads of {width} exceed {WIDE_ATTEND_MAX_WIDTH}")
+    if max_context > block_tables.shape[1] * bs:
+        raise KernelError("attention: block tables are shorter than the longest context")
+    call("as_wide_attend", _ptr(q), _ptr(k_pages), _ptr(v_pages), _DT[q.dtype], _ptr(positions), _ptr(tok_row),
+         _ptr(block_tables), block_tables.shape[1], _ptr(out), H, width, bs, float(scale), T, _stream())

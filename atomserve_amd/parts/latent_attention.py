@@ -37,9 +37,13 @@ class LatentAttention(Mixer):
         widest = s.kv_rank + s.rot_dim
         # what the attention kernels take as a head: multiples of 32 on the matrix cores, else of the chunk they load
         self.width = -(-widest // 32) * 32 if widest > 16 else -(-widest // chunk) * chunk
-        if self.width > ops.SINGLE_QUERY_MAX_HEAD_DIM:
+        # a page wider than those kernels' heads goes through a kernel of its own, plain and for any width
+        self.wide = self.width > ops.SINGLE_QUERY_MAX_HEAD_DIM
+        if self.wide:
+            self.width = -(-widest // chunk) * chunk
+        if self.width > ops.WIDE_ATTEND_MAX_WIDTH or s.kv_rank > ops.LATENT_MAX_RANK or s.head_dim > ops.LATENT_MAX_HEAD_DIM:
             raise ValueError(f"a latent of {s.kv_rank} and a turned part of {s.rot_dim} exceed the attention kernels' heads "
-                             f"of {ops.SINGLE_QUERY_MAX_HEAD_DIM}")  # fmt: skip
+                             f"of {ops.WIDE_ATTEND_MAX_WIDTH}")  # fmt: skip
         self.dkv_off = s.q_rank
         self.g_off = s.q_rank + (widest if s.own_latent else 0)
         self.in_rows = self.g_off + s.num_heads * s.value_dim
@@ -83,7 +87,7 @@ class LatentAttention(Mixer):
         return PagedCacheRequest(1, self.width, 0)
 
     def row_split(self):
-        return (SHORT_ROW, TILE_Q)
+        return None if self.wide else (SHORT_ROW, TILE_Q)
 
     def forward(self, h, step, cache):
         s, env = self.spec, self.env
@@ -102,7 +106,11 @@ class LatentAttention(Mixer):
         qa = torch.empty((T, H, self.width), dtype=env.dtype, device=dev)
         ops.latent_q_absorb(q, self.uk_weight, H, D, R, s.kv_rank, cos_sin, qa)
         heads = torch.empty((T, H, self.width), dtype=env.dtype, device=dev)
-        attend(qa, heads, step, cache, s.scale, 0, self.row_split())
+        if self.wide:
+            ops.wide_attend(qa, cache.k_pages, cache.v_pages, step.positions, None if step.decode_only else step.tok_row,
+                            cache.block_tables, heads, s.scale, step.max_context)  # fmt: skip
+        else:
+            attend(qa, heads, step, cache, s.scale, 0, self.row_split())
         act = torch.empty((T, H * E), dtype=env.dtype, device=dev)
         ops.latent_v_expand(heads, self.uv_t, s.kv_rank, proj, self.g_off, act)
         y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=dev)

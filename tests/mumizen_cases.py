@@ -66,6 +66,24 @@ CASES = {
             {"type": "latent_attention", "mixer": _latent(6, 16, 2, 8, 8, 56, 0.25, 7.0, (2.0, 16, 4.0, 0.5)), "mlp": _dense(24, 6.0)},
         ],
     },  # fmt: skip
+    # a latent wider than the paged attention kernels' heads, with a reader; a rotation over few coordinates
+    "wide_latent": {
+        "architecture": "Mumizen", "vocab": 150, "width": 64, "norm": {"eps": 1e-5, "groups": 2},
+        "layers": [
+            {"type": "latent_attention", "mixer": _latent(2, 16, 4, 24, 16, 270, 0.06, 300.0, (4.0, 32, 8.0, 1.0)), "mlp": _dense(32, 2.0)},
+            {"type": "latent_attention", "mixer": _latent(3, 8, 4, 8, 24, 270, 0.08, 300.0, (4.0, 32, 8.0, 1.0), kv_from=0), "mlp": None},
+        ],
+    },  # fmt: skip
+    # sizes that are multiples of nothing: odd vocabulary, heads of 10 and 14, latents of 20 and 36, inner widths of 20 and 12
+    "odd_sizes": {
+        "architecture": "Mumizen", "vocab": 203, "width": 88, "norm": {"eps": 1e-6, "groups": 2},
+        "layers": [
+            {"type": "retention", "mixer": _decay(3, 10, 14, (0.99, 0.9, 0.75)), "mlp": _dense(20, 1.0)},
+            {"type": "latent_attention", "mixer": _latent(3, 10, 6, 10, 20, 36, 0.25, 1000.0, (8.0, 32, 32.0, 1.0)), "mlp": _moe(12, 1.5, 6, 3, (20, 2.0))},
+            {"type": "lightning", "mixer": _decay(5, 6, 6, (0.6, 0.8, 0.9, 0.97, 0.999)), "mlp": _moe(12, 1.5, 4, 2)},
+            {"type": "latent_attention", "mixer": _latent(7, 6, 6, 10, 12, 36, 0.3, 1000.0, (8.0, 32, 32.0, 1.0), kv_from=1), "mlp": _dense(28, 2.0)},
+        ],
+    },  # fmt: skip
 }
 
 

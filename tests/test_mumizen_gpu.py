@@ -568,6 +568,35 @@ def test_attention_through_a_latent(shape, dtype):
         assert (got - want).abs().max() <= tol, f"{shape} pages of {bs}: {float((got - want).abs().max()):.3e} of {float(want.abs().max()):.3e}"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(3, 8, 8, 16, 300, 16), (2, 24, 2, 8, 514, 4), (5, 8, 4, 8, 40, 64)])
+def test_attention_over_a_wide_latent(shape, dtype):
+    """The kernel for pages wider than the paged attention kernels' heads (and any narrower ones) against the plain
+    form: 600 positions (three blocks of keys), a far latent that every query matches from position 280 on."""
+    from atomserve_amd.kernels import ops
+
+    H, D, R, E, rank, bs = shape
+    L, gen = 600, torch.Generator().manual_seed(sum(shape))
+    t = DTYPES[dtype]
+    q, c, kr = bf(torch.randn(L, H, D + R, generator=gen)), bf(torch.randn(L, rank, generator=gen)), bf(torch.randn(L, R, generator=gen))
+    uk, uv = bf(0.3 * torch.randn(H * D, rank, generator=gen)), bf(0.3 * torch.randn(H * E, rank, generator=gen))
+    c[280] *= 3.0
+    want = plain_latent_attention(q.double(), c.double(), kr.double(), uk.double(), uv.double(), 0.05).float()
+    width = -(-(rank + R) // 8) * 8
+    kp, vp, table = latent_pages(c, kr, bs, width, gen, dtype, junk=3.0)
+    ones = torch.zeros(L, R // 2, 2)
+    ones[..., 0] = 1.0
+    qa = torch.empty((L, H, width), dtype=t, device=DEV)
+    ops.latent_q_absorb(dev(q.reshape(L, -1), t), dev(uk, t), H, D, R, rank, dev(ones), qa)
+    heads = torch.zeros((L, H, width), dtype=t, device=DEV)
+    ops.wide_attend(qa, kp, vp, torch.arange(L, dtype=I32, device=DEV), torch.zeros(L, dtype=I32, device=DEV), table, heads, 0.05, L)
+    out = torch.empty((L, H * E), dtype=t, device=DEV)
+    ops.latent_v_expand(heads, dev(uv.view(H, E, rank).transpose(1, 2), t), rank, None, 0, out)
+    got = out.float().cpu().view(L, H, E)
+    tol = (3e-5 if dtype == "float32" else 3e-2) * float(want.abs().max())
+    assert (got - want).abs().max() <= tol, f"{shape}: {float((got - want).abs().max()):.3e} of {float(want.abs().max()):.3e}"
+
+
 @pytest.mark.parametrize("block_size", [8, 16, 64])
 def test_a_far_latent_and_pages_borders_show(block_size):
     """One cached latent that every head's query matches far better than any other: from its position on every
