@@ -229,14 +229,14 @@ extern "C" int as_rmsnorm_split(float* x, const float* sums, int splits, int num
 // range reduction are done in fp64 so that large positions keep fp32-exact angles;
 // the rotation itself is fp32.  Plain reference: reference atomserve/model.py:142-169.
 __global__ void rope_table_kernel(const int* __restrict__ positions, const double* __restrict__ inv_freq,
-                                  float2* __restrict__ cs, int num_tokens, int half) {
+                                  float2* __restrict__ cs, int num_tokens, int half, float magnitude) {
   const int idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= num_tokens * half) return;
   const int t = idx / half, i = idx % half;
   const double a = (double)positions[t] * inv_freq[i];
   double s, c;
   sincos(a, &s, &c);
-  cs[idx] = make_float2((float)c, (float)s);
+  cs[idx] = make_float2((float)c * magnitude, (float)s * magnitude);
 }
 
 extern "C" int as_rope_table(const int* positions, const double* inv_freq, float* cs, int num_tokens,
@@ -244,7 +244,17 @@ extern "C" int as_rope_table(const int* positions, const double* inv_freq, float
   if (num_tokens <= 0) return AS_OK;
   if (half <= 0) return AS_BAD_SHAPE;
   const int total = num_tokens * half;
-  rope_table_kernel<<<(total + 255) / 256, 256, 0, stream>>>(positions, inv_freq, (float2*)cs, num_tokens, half);
+  rope_table_kernel<<<(total + 255) / 256, 256, 0, stream>>>(positions, inv_freq, (float2*)cs, num_tokens, half, 1.0f);
+  return launch_status();
+}
+
+// The same with cosines and sines multiplied by `magnitude` (rotations stretched for long contexts).
+extern "C" int as_rope_table_scaled(const int* positions, const double* inv_freq, float* cs, int num_tokens,
+                                    int half, float magnitude, hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (half <= 0) return AS_BAD_SHAPE;
+  const int total = num_tokens * half;
+  rope_table_kernel<<<(total + 255) / 256, 256, 0, stream>>>(positions, inv_freq, (float2*)cs, num_tokens, half, magnitude);
   return launch_status();
 }
 

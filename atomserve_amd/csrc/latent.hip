@@ -13,7 +13,7 @@
 //   latent_v_expand   heads [T, H, width] (their first kv_rank coordinates) -> V_h heads, times sigmoid(gate)
 //   wide_attend       the attention itself for latents wider than the paged attention kernels' heads
 //
-// Norms, the rotation and every sum are fp32; an output is one chain of multiply-adds in a fixed order.
+// Norms, the rotation and every sum are fp32, taken in an order that does not depend on what else is in the step.
 #include "common.h"
 
 template <typename T>
@@ -93,115 +93,194 @@ extern "C" int as_latent_kv_store(const void* proj, int dtype, int ld, int off, 
   return launch_status();
 }
 
-// q [T, H, D + R]; uk [H * D, rank] (row h D + d: what coordinate d of head h's keys reads of the latent).
-// out [T, H, width]: out[t, h, r] = sum_d q[t, h, d] uk[h D + d, r] for r < rank, then the R rotated coordinates
-// of q, then zeros.  grid (token tiles of ABSORB_TOKENS, heads).
+// ---- products with a matrix per head --------------------------------------------------------------------------
+// out[t, h, n] = sum_k x[t, h, k] W_h[k, n] for two uses: the queries' plain part through U_h (k a coordinate of the
+// head, n one of the latent) and the attention's result through V_h (k a coordinate of the latent, n one of the
+// value).  Few tokens: `head_product_kernel`, any dtype, W_h stored [k][n]; a workgroup owns 64 outputs of a head for
+// up to 8 tokens, its four waves a quarter of k each, and the four partial sums are added in the waves' order.
+// Prompts in bfloat16: `head_product_mfma_kernel`, W_h stored [n][k], on the matrix cores (weights as the first
+// operand, 16 tokens as the second: a lane then holds four consecutive outputs of one token).
 #define ABSORB_TOKENS 8
+#define HEAD_STRIP 64  // outputs a workgroup owns
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// What follows the product.  TAIL (the queries): out[t, h, N .. N + R) = the R coordinates after the K plain ones
+// of x[t, h], turned by cos_sin [T, R/2, 2], then zeros up to `os`.  GATE (the values): the product rounded as it
+// would be stored, times sigmoid(gate[t, g_off + h N + n]) (gate null: none).
+struct HeadEpilogue {
+  int R;
+  const float* cos_sin;
+  const void* gate;
+  int ld, g_off;
+};
+
+template <typename T, bool GATE>
+__device__ __forceinline__ void head_store(float v, size_t t, int h, int n, int N, int H, T* __restrict__ out, int os,
+                                           const HeadEpilogue& ep) {
+  if (GATE) {
+    if (ep.gate) {
+      v = to_f32(from_f32<T>(v));
+      v *= 1.0f / (1.0f + expf(-to_f32(((const T*)ep.gate)[t * ep.ld + ep.g_off + h * N + n])));
+    }
+  }
+  out[(t * H + h) * os + n] = from_f32<T>(v);
+}
 
 template <typename T>
-__global__ __launch_bounds__(256) void latent_q_absorb_kernel(const T* __restrict__ q, const T* __restrict__ uk, int H,
-                                                              int D, int R, int rank, const float* __restrict__ cos_sin,
-                                                              T* __restrict__ out, int width, int num_tokens) {
-  extern __shared__ float qs[];  // [ABSORB_TOKENS][D]
-  const int t0 = blockIdx.x * ABSORB_TOKENS, h = blockIdx.y;
-  const int nt = min(ABSORB_TOKENS, num_tokens - t0);
-  for (int i = threadIdx.x; i < ABSORB_TOKENS * D; i += blockDim.x) {
-    const int tq = i / D, d = i % D;
-    qs[i] = tq < nt ? to_f32(q[((size_t)(t0 + tq) * H + h) * (D + R) + d]) : 0.f;
-  }
-  __syncthreads();
-  const T* w = uk + (size_t)h * D * rank;
-  for (int r = threadIdx.x; r < rank; r += blockDim.x) {
-    float acc[ABSORB_TOKENS];
-#pragma unroll
-    for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = 0.f;
-    for (int d = 0; d < D; ++d) {
-      const float wv = to_f32(w[(size_t)d * rank + r]);
-#pragma unroll
-      for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = fmaf(qs[tq * D + d], wv, acc[tq]);
-    }
-    for (int tq = 0; tq < nt; ++tq) out[((size_t)(t0 + tq) * H + h) * width + r] = from_f32<T>(acc[tq]);
-  }
-  const int half = R / 2, tail = width - rank;
+__device__ __forceinline__ void head_tail(const T* __restrict__ x, int xs, int K, int N, int H, int h, int t0, int nt,
+                                          T* __restrict__ out, int os, const HeadEpilogue& ep) {
+  const int half = ep.R / 2, tail = os - N;
   for (int i = threadIdx.x; i < nt * tail; i += blockDim.x) {
-    const int tq = i / tail, j = i % tail, t = t0 + tq;
+    const int tq = i / tail, j = i % tail;
+    const size_t t = t0 + tq;
     float v = 0.f;
-    if (j < R) {
+    if (j < ep.R) {
       const int p = j < half ? j : j - half;
-      const T* qr = q + ((size_t)t * H + h) * (D + R) + D;
-      const float c = cos_sin[((size_t)t * half + p) * 2], s = cos_sin[((size_t)t * half + p) * 2 + 1];
-      const float a = to_f32(qr[p]), b = to_f32(qr[half + p]);
+      const T* xr = x + (t * H + h) * xs + K;
+      const float c = ep.cos_sin[(t * half + p) * 2], s = ep.cos_sin[(t * half + p) * 2 + 1];
+      const float a = to_f32(xr[p]), b = to_f32(xr[half + p]);
       v = j < half ? a * c - b * s : b * c + a * s;
     }
-    out[((size_t)t * H + h) * width + rank + j] = from_f32<T>(v);
+    out[(t * H + h) * os + N + j] = from_f32<T>(v);
   }
 }
 
-extern "C" int as_latent_q_absorb(const void* q, const void* uk, int dtype, int H, int D, int R, int rank,
-                                  const float* cos_sin, void* out, int width, int num_tokens, hipStream_t stream) {
+// x [T, H, xs] (the first K of a row count), w [H, K, N], out [T, H, os].  grid (token tiles of ABSORB_TOKENS, heads,
+// strips of HEAD_STRIP outputs).
+template <typename T, bool GATE>
+__global__ __launch_bounds__(256) void head_product_kernel(const T* __restrict__ x, int xs, const T* __restrict__ w,
+                                                           int K, int N, int H, int num_tokens, T* __restrict__ out,
+                                                           int os, HeadEpilogue ep) {
+  extern __shared__ float lds[];  // [ABSORB_TOKENS][K] the inputs, [4][ABSORB_TOKENS][HEAD_STRIP] the waves' sums
+  float* xl = lds;
+  float* part = lds + ABSORB_TOKENS * K;
+  const int t0 = blockIdx.x * ABSORB_TOKENS, h = blockIdx.y, n0 = blockIdx.z * HEAD_STRIP;
+  const int nt = min(ABSORB_TOKENS, num_tokens - t0);
+  for (int i = threadIdx.x; i < ABSORB_TOKENS * K; i += blockDim.x) {
+    const int tq = i / K, k = i % K;
+    xl[i] = tq < nt ? to_f32(x[((size_t)(t0 + tq) * H + h) * xs + k]) : 0.f;
+  }
+  __syncthreads();
+  const int nl = threadIdx.x & 63, slice = threadIdx.x >> 6, n = n0 + nl;
+  const int per = (K + 3) / 4, k_lo = slice * per, k_hi = min(K, k_lo + per);
+  float acc[ABSORB_TOKENS];
+#pragma unroll
+  for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = 0.f;
+  if (n < N) {
+    const T* wh = w + (size_t)h * K * N + n;
+#pragma unroll 4
+    for (int k = k_lo; k < k_hi; ++k) {
+      const float wv = to_f32(wh[(size_t)k * N]);
+#pragma unroll
+      for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = fmaf(xl[tq * K + k], wv, acc[tq]);
+    }
+  }
+#pragma unroll
+  for (int tq = 0; tq < ABSORB_TOKENS; ++tq) part[(slice * ABSORB_TOKENS + tq) * HEAD_STRIP + nl] = acc[tq];
+  __syncthreads();
+  for (int i = threadIdx.x; i < nt * HEAD_STRIP; i += blockDim.x) {
+    const int tq = i / HEAD_STRIP, c = i % HEAD_STRIP;
+    if (n0 + c >= N) continue;
+    const float v = ((part[(0 * ABSORB_TOKENS + tq) * HEAD_STRIP + c] + part[(1 * ABSORB_TOKENS + tq) * HEAD_STRIP + c]) +
+                     part[(2 * ABSORB_TOKENS + tq) * HEAD_STRIP + c]) + part[(3 * ABSORB_TOKENS + tq) * HEAD_STRIP + c];
+    head_store<T, GATE>(v, t0 + tq, h, n0 + c, N, H, out, os, ep);
+  }
+  if (!GATE && blockIdx.z == 0) head_tail<T>(x, xs, K, N, H, h, t0, nt, out, os, ep);
+}
+
+// bfloat16, K % 32 == 0, xs % 8 == 0: w [H, N, K].  grid (token tiles of 128, heads, strips of HEAD_STRIP outputs); a
+// wave owns 32 tokens.
+#define MFMA_TOKENS 128
+template <bool GATE>
+__global__ __launch_bounds__(256) void head_product_mfma_kernel(const bf16* __restrict__ x, int xs,
+                                                                const bf16* __restrict__ w, int K, int N, int H,
+                                                                int num_tokens, bf16* __restrict__ out, int os,
+                                                                HeadEpilogue ep) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lr = lane & 15, lg = lane >> 4;
+  const int t0 = blockIdx.x * MFMA_TOKENS, h = blockIdx.y, n0 = blockIdx.z * HEAD_STRIP;
+  const int tw = t0 + wave * 32;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  floatx4 acc[2][4];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) acc[tt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    bf16x8 b[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const int t = tw + tt * 16 + lr;
+      b[tt] = t < num_tokens ? *reinterpret_cast<const bf16x8*>(x + ((size_t)t * H + h) * xs + k0 + lg * 8) : zero;
+    }
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int n = n0 + nt * 16 + lr;
+      const bf16x8 a = n < N ? *reinterpret_cast<const bf16x8*>(w + ((size_t)h * N + n) * K + k0 + lg * 8) : zero;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) acc[tt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[tt], acc[tt][nt], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    const int t = tw + tt * 16 + lr;
+    if (t >= num_tokens) continue;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + nt * 16 + 4 * lg + i;
+        if (n < N) head_store<bf16, GATE>(acc[tt][nt][i], (size_t)t, h, n, N, H, out, os, ep);
+      }
+  }
+  if (!GATE && blockIdx.z == 0) head_tail<bf16>(x, xs, K, N, H, h, t0, min(MFMA_TOKENS, num_tokens - t0), out, os, ep);
+}
+
+template <bool GATE>
+static int launch_head_product(const void* x, int xs, const void* w, const void* w_nk, int dtype, int K, int N, int H,
+                               int num_tokens, void* out, int os, const HeadEpilogue& ep, hipStream_t stream) {
+  const int strips = (N + HEAD_STRIP - 1) / HEAD_STRIP;
+  if (dtype == DT_BF16 && w_nk && num_tokens >= 32 && K % 32 == 0 && xs % 8 == 0) {
+    dim3 grid((num_tokens + MFMA_TOKENS - 1) / MFMA_TOKENS, H, strips);
+    head_product_mfma_kernel<GATE><<<grid, 256, 0, stream>>>((const bf16*)x, xs, (const bf16*)w_nk, K, N, H, num_tokens, (bf16*)out, os, ep);
+    return launch_status();
+  }
+  dim3 grid((num_tokens + ABSORB_TOKENS - 1) / ABSORB_TOKENS, H, strips);
+  const size_t lds = (size_t)ABSORB_TOKENS * (K + 4 * HEAD_STRIP) * sizeof(float);
+  if (lds > (64u << 10)) return AS_BAD_SHAPE;
+  if (dtype == DT_F32)
+    head_product_kernel<float, GATE><<<grid, 256, lds, stream>>>((const float*)x, xs, (const float*)w, K, N, H, num_tokens, (float*)out, os, ep);
+  else if (dtype == DT_BF16)
+    head_product_kernel<bf16, GATE><<<grid, 256, lds, stream>>>((const bf16*)x, xs, (const bf16*)w, K, N, H, num_tokens, (bf16*)out, os, ep);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// q [T, H, D + R]; uk [H * D, rank] (row h D + d: what coordinate d of head h's keys reads of the latent), uk_t
+// [H, rank, D] the same transposed (null: none; bfloat16 prompts then run the general kernel).
+// out [T, H, width]: out[t, h, r] = sum_d q[t, h, d] uk[h D + d, r] for r < rank, then the R rotated coordinates
+// of q, then zeros.
+extern "C" int as_latent_q_absorb(const void* q, const void* uk, const void* uk_t, int dtype, int H, int D, int R,
+                                  int rank, const float* cos_sin, void* out, int width, int num_tokens,
+                                  hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
   if (H <= 0 || H > 65535 || D <= 0 || R < 0 || R % 2 || rank <= 0 || rank + R > width || D > 1024) return AS_BAD_SHAPE;
   if (R > 0 && !cos_sin) return AS_BAD_SHAPE;
-  dim3 grid((num_tokens + ABSORB_TOKENS - 1) / ABSORB_TOKENS, H);
-  const size_t lds = (size_t)ABSORB_TOKENS * D * sizeof(float);
-  if (dtype == DT_F32)
-    latent_q_absorb_kernel<float><<<grid, 256, lds, stream>>>((const float*)q, (const float*)uk, H, D, R, rank, cos_sin, (float*)out, width, num_tokens);
-  else if (dtype == DT_BF16)
-    latent_q_absorb_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)uk, H, D, R, rank, cos_sin, (bf16*)out, width, num_tokens);
-  else return AS_BAD_DTYPE;
-  return launch_status();
+  const HeadEpilogue ep = {R, cos_sin, nullptr, 0, 0};
+  return launch_head_product<false>(q, D + R, uk, uk_t, dtype, D, rank, H, num_tokens, out, width, ep, stream);
 }
 
 // heads [T, H, width]: what the attention over the latent left per head (its first `rank` coordinates count).
-// uv_t [H, rank, E]: head h's value matrix, transposed.  out[t, h E + e] = (sum_r heads[t, h, r] uv_t[h, r, e]) *
-// sigmoid(gate[t, g_off + h E + e]) (gate null: no gate).  grid (token tiles of ABSORB_TOKENS, heads).
-template <typename T>
-__global__ __launch_bounds__(256) void latent_v_expand_kernel(const T* __restrict__ heads, const T* __restrict__ uv_t,
-                                                              int H, int E, int rank, int width,
-                                                              const T* __restrict__ gate, int ld, int g_off,
-                                                              T* __restrict__ out, int num_tokens) {
-  extern __shared__ float os[];  // [ABSORB_TOKENS][rank]
-  const int t0 = blockIdx.x * ABSORB_TOKENS, h = blockIdx.y;
-  const int nt = min(ABSORB_TOKENS, num_tokens - t0);
-  for (int i = threadIdx.x; i < ABSORB_TOKENS * rank; i += blockDim.x) {
-    const int tq = i / rank, r = i % rank;
-    os[i] = tq < nt ? to_f32(heads[((size_t)(t0 + tq) * H + h) * width + r]) : 0.f;
-  }
-  __syncthreads();
-  const T* w = uv_t + (size_t)h * rank * E;
-  for (int e = threadIdx.x; e < E; e += blockDim.x) {
-    float acc[ABSORB_TOKENS];
-#pragma unroll
-    for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = 0.f;
-    for (int r = 0; r < rank; ++r) {
-      const float wv = to_f32(w[(size_t)r * E + e]);
-#pragma unroll
-      for (int tq = 0; tq < ABSORB_TOKENS; ++tq) acc[tq] = fmaf(os[tq * rank + r], wv, acc[tq]);
-    }
-    for (int tq = 0; tq < nt; ++tq) {
-      const size_t t = t0 + tq;
-      float v = acc[tq];
-      if (gate) {
-        v = to_f32(from_f32<T>(v));  // the head's value as it would be stored
-        v *= 1.0f / (1.0f + expf(-to_f32(gate[t * ld + g_off + h * E + e])));
-      }
-      out[(t * H + h) * E + e] = from_f32<T>(v);
-    }
-  }
-}
-
-extern "C" int as_latent_v_expand(const void* heads, const void* uv_t, int dtype, int H, int E, int rank, int width,
-                                  const void* gate, int ld, int g_off, void* out, int num_tokens, hipStream_t stream) {
+// uv_t [H, rank, E]: head h's value matrix, transposed; uv [H * E, rank] as the checkpoint holds it (null: none).
+// out[t, h E + e] = (sum_r heads[t, h, r] uv_t[h, r, e]) * sigmoid(gate[t, g_off + h E + e]) (gate null: no gate).
+extern "C" int as_latent_v_expand(const void* heads, const void* uv_t, const void* uv, int dtype, int H, int E,
+                                  int rank, int width, const void* gate, int ld, int g_off, void* out,
+                                  int num_tokens, hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
-  if (H <= 0 || H > 65535 || E <= 0 || rank <= 0 || rank > width || rank > 4096) return AS_BAD_SHAPE;
-  dim3 grid((num_tokens + ABSORB_TOKENS - 1) / ABSORB_TOKENS, H);
-  const size_t lds = (size_t)ABSORB_TOKENS * rank * sizeof(float);
-  if (dtype == DT_F32)
-    latent_v_expand_kernel<float><<<grid, 256, lds, stream>>>((const float*)heads, (const float*)uv_t, H, E, rank, width, (const float*)gate, ld, g_off, (float*)out, num_tokens);
-  else if (dtype == DT_BF16)
-    latent_v_expand_kernel<bf16><<<grid, 256, lds, stream>>>((const bf16*)heads, (const bf16*)uv_t, H, E, rank, width, (const bf16*)gate, ld, g_off, (bf16*)out, num_tokens);
-  else return AS_BAD_DTYPE;
-  return launch_status();
+  if (H <= 0 || H > 65535 || E <= 0 || rank <= 0 || rank > width || rank > 1536) return AS_BAD_SHAPE;
+  const HeadEpilogue ep = {0, nullptr, gate, ld, g_off};
+  return launch_head_product<true>(heads, width, uv_t, uv, dtype, rank, E, H, num_tokens, out, E, ep, stream);
 }
 
 // ---- attention over one kv head of any width ------------------------------------------------------------------

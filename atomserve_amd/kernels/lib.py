@@ -22,6 +22,7 @@ SIGNATURES = {
     "as_rmsnorm": ("elementwise", [P, P, P, P, I, F, P, I, I, I, I, P]),
     "as_rmsnorm_split": ("elementwise", [P, P, I, I, P, P, I, F, P, I, I, I, I, P]),
     "as_rope_table": ("elementwise", [P, P, P, I, I, P]),
+    "as_rope_table_scaled": ("elementwise", [P, P, P, I, I, F, P]),
     "as_qk_norm_rope_store": ("elementwise", [P, I, P, P, I, P, P, P, P, P, I, I, I, I, I, F, I, I, P]),
     "as_silu_mul": ("elementwise", [P, P, I, I, I, P]),
     "as_rmsnorm_multi": ("elementwise", [P, P, P, P, P, P, I, F, P, P, I, I, I, I, P]),
@@ -48,8 +49,8 @@ SIGNATURES = {
     "as_decay_finish": ("linear_attention", [P, I, I, F, P, P, I, I, I, I, P, I, P]),
     "as_rows_rms_norm": ("latent", [P, I, I, I, I, P, F, P, I, P]),
     "as_latent_kv_store": ("latent", [P, I, I, I, I, I, P, F, P, P, P, P, I, I, I, P]),
-    "as_latent_q_absorb": ("latent", [P, P, I, I, I, I, I, P, P, I, I, P]),
-    "as_latent_v_expand": ("latent", [P, P, I, I, I, I, I, P, I, I, P, I, P]),
+    "as_latent_q_absorb": ("latent", [P, P, P, I, I, I, I, I, P, P, I, I, P]),
+    "as_latent_v_expand": ("latent", [P, P, P, I, I, I, I, I, P, I, I, P, I, P]),
     "as_wide_attend": ("latent", [P, P, P, I, P, P, P, I, P, I, I, I, F, I, P]),
     "as_attn_headmix_mfma": ("attention_mix", [P, P, P, P, I, I, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, I, P, P, P]),
     "as_attn_headmix": ("attention_mix", [P, P, P, I, P, I, I, P, P, P, I, P, P, I, I, I, I, I, F, I, I, P]),

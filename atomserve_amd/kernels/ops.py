@@ -146,12 +146,16 @@ def rmsnorm(x, weight, eps, out, delta=None, rows=None, update_x=True, split_sum
          _DT[out.dtype], n_out, n, int(bool(update_x)), _stream())  # fmt: skip
 
 
-def rope_table(positions, inv_freq, out) -> None:
-    """out[t, i] = (cos, sin)(positions[t] * inv_freq[i]); inv_freq fp64 [R/2], out fp32 [T, R/2, 2]."""
+def rope_table(positions, inv_freq, out, magnitude: float = 1.0) -> None:
+    """out[t, i] = magnitude * (cos, sin)(positions[t] * inv_freq[i]); inv_freq fp64 [R/2], out fp32 [T, R/2, 2]."""
     _check(positions, "positions", I32, (None,))
     _check(inv_freq, "inv_freq", torch.float64, (None,))
     _check(out, "out", F32, (positions.shape[0], inv_freq.shape[0], 2))
-    call("as_rope_table", _ptr(positions), _ptr(inv_freq), _ptr(out), positions.shape[0], inv_freq.shape[0], _stream())
+    if magnitude == 1.0:
+        call("as_rope_table", _ptr(positions), _ptr(inv_freq), _ptr(out), positions.shape[0], inv_freq.shape[0], _stream())
+    else:
+        call("as_rope_table_scaled", _ptr(positions), _ptr(inv_freq), _ptr(out), positions.shape[0], inv_freq.shape[0],
+             float(magnitude), _stream())  # fmt: skip
 
 
 def qk_norm_rope_store(qkv, q_weight, k_weight, cos_sin, slots, q_out, k_pages, v_pages, num_heads,
@@ -1724,28 +1728,34 @@ def latent_kv_store(proj, off, rank, rot, gain, eps, cos_sin, slots, k_pages, v_
          _ptr(slots), _ptr(k_pages), _ptr(v_pages), bs, width, T, _stream())  # fmt: skip
 
 
-def latent_q_absorb(q, uk, num_heads, dim, rot, rank, cos_sin, out) -> None:
+def latent_q_absorb(q, uk, num_heads, dim, rot, rank, cos_sin, out, uk_t=None) -> None:
     """q [T, heads * (dim + rot)], uk [heads * dim, rank]: out[t, h] = [uk_h^T q_h[:dim] | q_h[dim:] turned by
-    cos_sin | zeros]; out [T, heads, width]."""
+    cos_sin | zeros]; out [T, heads, width].  uk_t [heads, rank, dim]: the same matrices transposed, with which
+    bfloat16 prompts multiply on the matrix cores."""
     _check(q, "q", (F32, BF16), (None, num_heads * (dim + rot)))
     T = q.shape[0]
     _check(uk, "uk", q.dtype, (num_heads * dim, rank))
+    if uk_t is not None:
+        _check(uk_t, "uk_t", q.dtype, (num_heads, rank, dim))
     _check(out, "out", q.dtype, (T, num_heads, None))
     if rot:
         _check(cos_sin, "cos_sin", F32, (T, rot // 2, 2))
-    if rank + rot > out.shape[2] or rot % 2:
-        raise KernelError("latent_q_absorb: the latent and the turned part exceed the output's width")
-    call("as_latent_q_absorb", _ptr(q), _ptr(uk), _DT[q.dtype], num_heads, dim, rot, rank, _ptr(cos_sin), _ptr(out),
-         out.shape[2], T, _stream())  # fmt: skip
+    if rank + rot > out.shape[2] or rot % 2 or dim > LATENT_MAX_HEAD_DIM:
+        raise KernelError("latent_q_absorb: the latent and the turned part exceed the output's width, or the heads the kernel's")
+    call("as_latent_q_absorb", _ptr(q), _ptr(uk), _ptr(uk_t), _DT[q.dtype], num_heads, dim, rot, rank, _ptr(cos_sin),
+         _ptr(out), out.shape[2], T, _stream())  # fmt: skip
 
 
-def latent_v_expand(heads, uv_t, rank, gate, g_off, out) -> None:
+def latent_v_expand(heads, uv_t, rank, gate, g_off, out, uv=None) -> None:
     """heads [T, H, width] (the first `rank` coordinates count), uv_t [H, rank, E]: out[t, h E + e] = (sum_r heads[t, h,
-    r] uv_t[h, r, e]) * sigmoid(gate[t, g_off + h E + e]); gate [T, ld] or None (no gate); out [T, H * E]."""
+    r] uv_t[h, r, e]) * sigmoid(gate[t, g_off + h E + e]); gate [T, ld] or None (no gate); out [T, H * E].  uv [H * E,
+    rank]: the same matrices as a checkpoint holds them, with which bfloat16 prompts multiply on the matrix cores."""
     _check(heads, "heads", (F32, BF16), (None, None, None))
     T, H, width = heads.shape
     _check(uv_t, "uv_t", heads.dtype, (H, rank, None))
     E = uv_t.shape[2]
+    if uv is not None:
+        _check(uv, "uv", heads.dtype, (H * E, rank))
     _check(out, "out", heads.dtype, (T, H * E))
     ld = 0
     if gate is not None:
@@ -1753,10 +1763,10 @@ def latent_v_expand(heads, uv_t, rank, gate, g_off, out) -> None:
         ld = gate.shape[1]
         if g_off < 0 or g_off + H * E > ld:
             raise KernelError("latent_v_expand: the gate's columns lie outside its rows")
-    if rank > width:
-        raise KernelError("latent_v_expand: the latent is wider than the heads")
-    call("as_latent_v_expand", _ptr(heads), _ptr(uv_t), _DT[heads.dtype], H, E, rank, width, _ptr(gate), ld, g_off,
-         _ptr(out), T, _stream())  # fmt: skip
+    if rank > width or rank > LATENT_MAX_RANK:
+        raise KernelError("latent_v_expand: the latent is wider than the heads, or than the kernel takes")
+    call("as_latent_v_expand", _ptr(heads), _ptr(uv_t), _ptr(uv), _DT[heads.dtype], H, E, rank, width, _ptr(gate), ld,
+         g_off, _ptr(out), T, _stream())  # fmt: skip
 
 
 WIDE_ATTEND_MAX_WIDTH = 2048

@@ -75,7 +75,8 @@ class LatentAttention(Mixer):
             self.kv_norm_weight = self.kv_norm_weight.float().contiguous()
         # every head's value matrix transposed, [heads, kv_rank, value_dim]: lanes that own neighbouring outputs read neighbours
         self.uv_t = self.uv_weight.view(s.num_heads, s.value_dim, s.kv_rank).transpose(1, 2).contiguous()
-        del self.uv_weight
+        # and every head's key matrix transposed, [heads, kv_rank, head_dim]: what prompts multiply with on the matrix cores
+        self.uk_t = self.uk_weight.view(s.num_heads, s.head_dim, s.kv_rank).transpose(1, 2).contiguous()
         self.inp = ops.Streamed(self.in_weight, self.env.stream_copies)
         self.uq = ops.Streamed(self.uq_weight, self.env.stream_copies)
         self.o = ops.Streamed(self.o_weight, self.env.stream_copies)
@@ -104,7 +105,7 @@ class LatentAttention(Mixer):
         q = torch.empty((T, H * (D + R)), dtype=env.dtype, device=dev)
         ops.gemm(cq, self.uq, q, env.products)
         qa = torch.empty((T, H, self.width), dtype=env.dtype, device=dev)
-        ops.latent_q_absorb(q, self.uk_weight, H, D, R, s.kv_rank, cos_sin, qa)
+        ops.latent_q_absorb(q, self.uk_weight, H, D, R, s.kv_rank, cos_sin, qa, uk_t=self.uk_t)
         heads = torch.empty((T, H, self.width), dtype=env.dtype, device=dev)
         if self.wide:
             ops.wide_attend(qa, cache.k_pages, cache.v_pages, step.positions, None if step.decode_only else step.tok_row,
@@ -112,7 +113,7 @@ class LatentAttention(Mixer):
         else:
             attend(qa, heads, step, cache, s.scale, 0, self.row_split())
         act = torch.empty((T, H * E), dtype=env.dtype, device=dev)
-        ops.latent_v_expand(heads, self.uv_t, s.kv_rank, proj, self.g_off, act)
+        ops.latent_v_expand(heads, self.uv_t, s.kv_rank, proj, self.g_off, act, uv=self.uv_weight)
         y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=dev)
         ops.gemm(act, self.o, y, env.products)
         return y

@@ -74,9 +74,7 @@ class ScaledRotaryHalf(Position):
         if table is None:
             table = torch.empty((step.num_tokens, self.spec.rotary_dim // 2, 2), dtype=torch.float32,
                                 device=self.env.device)  # fmt: skip
-            ops.rope_table(step.positions, self.inv_freq, table)
-            if self.magnitude != 1.0:
-                table.mul_(self.magnitude)
+            ops.rope_table(step.positions, self.inv_freq, table, self.magnitude)
             step.shared[key] = table
         return table
 

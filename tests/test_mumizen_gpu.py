@@ -525,7 +525,11 @@ def latent_attend(q, c, kr, uk, uv, scale, dtype, bs, gen, singles=True):
     ones = torch.zeros(L, max(R // 2, 1), 2)
     ones[..., 0] = 1.0  # cos 1, sin 0: the queries come turned
     qa = torch.empty((L, H, width), dtype=t, device=DEV)
-    ops.latent_q_absorb(dev(q.reshape(L, -1), t), dev(uk, t), H, D, R, rank, dev(ones) if R else None, qa)
+    uk_t = dev(uk.view(H, D, rank).transpose(1, 2), t)  # with it, bfloat16 prompts multiply on the matrix cores
+    ops.latent_q_absorb(dev(q.reshape(L, -1), t), dev(uk, t), H, D, R, rank, dev(ones) if R else None, qa, uk_t=uk_t)
+    few = torch.empty((5, H, width), dtype=t, device=DEV)  # and few tokens through the general kernel: the same
+    ops.latent_q_absorb(dev(q.reshape(L, -1)[40:45], t), dev(uk, t), H, D, R, rank, dev(ones[40:45]) if R else None, few, uk_t=uk_t)
+    assert (few.float() - qa[40:45].float()).abs().max() <= (1e-5 if dtype == "float32" else 2e-2) * float(qa.float().abs().max())
     heads = torch.zeros((L, H, width), dtype=t, device=DEV)
     positions = torch.arange(L, dtype=I32, device=DEV)
     rows = torch.zeros(L, dtype=I32, device=DEV)
@@ -536,7 +540,12 @@ def latent_attend(q, c, kr, uk, uv, scale, dtype, bs, gen, singles=True):
         ops.attn_prefill(qa, kp, vp, tiles, table, heads, scale, 0, L)
     out = torch.empty((L, H * E), dtype=t, device=DEV)
     uv_t = dev(uv.view(H, E, rank).transpose(1, 2), t)
-    ops.latent_v_expand(heads, uv_t, rank, None, 0, out)
+    ops.latent_v_expand(heads, uv_t, rank, None, 0, out, uv=dev(uv, t))
+    gate = bf(torch.randn(7, 3 + H * E, generator=gen))
+    gated = torch.empty((7, H * E), dtype=t, device=DEV)
+    ops.latent_v_expand(heads[50:57].contiguous(), uv_t, rank, dev(gate, t), 3, gated, uv=dev(uv, t))
+    want = out[50:57].float().cpu() * torch.sigmoid(gate[:, 3:])
+    assert (gated.float().cpu() - want).abs().max() <= (1e-5 if dtype == "float32" else 2e-2) * float(want.abs().max())
     return out.float().cpu().view(L, H, E)
 
 
@@ -553,7 +562,7 @@ def plain_latent_attention(q, c, kr, uk, uv, scale):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape", [(3, 8, 8, 16, 40), (18, 4, 4, 8, 24), (4, 32, 32, 32, 128), (2, 40, 0, 16, 64), (6, 16, 2, 8, 222),
-                                   (32, 24, 64, 16, 192), (48, 8, 16, 8, 80)])
+                                   (32, 24, 64, 16, 192), (48, 8, 16, 8, 80), (8, 64, 32, 40, 96)])
 def test_attention_through_a_latent(shape, dtype):
     """Random queries, latents and key parts: heads' keys and values written out from the latent in the plain form,
     absorbed into the queries and applied after the attention in the kernels; as single tokens and in tiles."""
