@@ -13,6 +13,24 @@
 // Sums of squares, the norm, the shift, the residual sum and the depth average are fp32 in both precisions.
 #include "common.h"
 
+// Four consecutive values at once (the address a multiple of 16 bytes for fp32, of 8 for bfloat16).
+__device__ __forceinline__ void load4(const float* p, float* v) {
+  const float4 r = *reinterpret_cast<const float4*>(p);
+  v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+}
+__device__ __forceinline__ void load4(const bf16* p, float* v) {
+  const uint2 r = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
+  v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(bf16* p, const float* v) {
+  bf16 b[4] = {from_f32<bf16>(v[0]), from_f32<bf16>(v[1]), from_f32<bf16>(v[2]), from_f32<bf16>(v[3])};
+  *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(b);
+}
+
 // ---- the grouped norm of one row ------------------------------------------------------------------
 // inv[g] = 1 / sqrt(mean over group g of (x + d)^2 + eps); the waves take the groups in turn, a group's sum meets
 // by lane swaps.  The caller synchronises before reading `inv`.
@@ -23,10 +41,24 @@ __device__ __forceinline__ void group_inverse_rms(const float* __restrict__ xr, 
   const int gs = n / groups;
   for (int g = wave; g < groups; g += waves) {
     float ss = 0.f;
-    for (int i = lane; i < gs; i += WAVE) {
-      float v = xr[g * gs + i];
-      if (dr) v += to_f32(dr[g * gs + i]);
-      ss = fmaf(v, v, ss);
+    if (gs % 4 == 0) {  // groups of a multiple of four: four values a load (rows start on 16 bytes)
+      for (int i = 4 * lane; i < gs; i += 4 * WAVE) {
+        float v[4], d[4];
+        load4(xr + g * gs + i, v);
+        if (dr) {
+          load4(dr + g * gs + i, d);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) v[c] += d[c];
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) ss = fmaf(v[c], v[c], ss);
+      }
+    } else {
+      for (int i = lane; i < gs; i += WAVE) {
+        float v = xr[g * gs + i];
+        if (dr) v += to_f32(dr[g * gs + i]);
+        ss = fmaf(v, v, ss);
+      }
     }
     ss = wave_sum(ss);
     if (lane == 0) inv[g] = 1.0f / sqrtf(ss / (float)gs + eps);
@@ -49,6 +81,24 @@ __global__ __launch_bounds__(256) void group_norm_kernel(float* __restrict__ x, 
   group_inverse_rms<O>(xr, dr, n, groups, eps, inv);
   __syncthreads();
   const int gs = n / groups;
+  if (gs % 4 == 0) {
+    for (int i = 4 * threadIdx.x; i < n; i += 4 * blockDim.x) {
+      float v[4], d[4], g[4];
+      load4(xr + i, v);
+      load4(w + i, g);
+      if (dr) {
+        load4(dr + i, d);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[c] += d[c];
+        if (update_x) store4(xr + i, v);
+      }
+      const float scale = inv[i / gs];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) v[c] = v[c] * scale * g[c];
+      store4(out + (size_t)r * n + i, v);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
     float v = xr[i];
     if (dr) {
@@ -92,6 +142,38 @@ __global__ __launch_bounds__(256) void group_norm_shift_kernel(const float* __re
   const int gs = n / groups;
   const bool from_slot = leads && row_start[r] > 0 && slot >= 0;
   float* kept = slot >= 0 ? state + (size_t)slot * n : nullptr;
+  if (gs % 4 == 0) {
+    for (int i = 4 * threadIdx.x; i < n; i += 4 * blockDim.x) {
+      float h[4], g[4], m[4], before[4] = {0.f, 0.f, 0.f, 0.f}, o[4];
+      load4(xr + i, h);
+      load4(w + i, g);
+      load4(mu + i, m);
+      const float scale = inv[i / gs];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) h[c] = h[c] * scale * g[c];
+      if (!leads) {
+        load4(xb + i, before);
+        const float sb = inv_before[i / gs];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) before[c] = before[c] * sb * g[c];
+      } else if (from_slot) {
+        load4(kept + i, before);
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) o[c] = h[c] + (before[c] - h[c]) * m[c];
+      store4(out + (size_t)t * n + i, o);
+      if (keeps) {  // read above by this same thread
+        if (last != t) {
+          load4(xl + i, h);
+          const float sl = inv_last[i / gs];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) h[c] = h[c] * sl * g[c];
+        }
+        store4(kept + i, h);
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
     const float h = xr[i] * inv[i / gs] * w[i];
     float before = 0.f;

@@ -11,6 +11,24 @@
 //   decay_finish  o normed in groups (per head, or all heads together) with an optional gain, times act(gate)
 #include "common.h"
 
+// Four consecutive values at once (the address a multiple of 16 bytes for fp32, of 8 for bfloat16).
+__device__ __forceinline__ void load4(const float* p, float* v) {
+  const float4 r = *reinterpret_cast<const float4*>(p);
+  v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w;
+}
+__device__ __forceinline__ void load4(const bf16* p, float* v) {
+  const uint2 r = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(r.x << 16); v[1] = __uint_as_float(r.x & 0xffff0000u);
+  v[2] = __uint_as_float(r.y << 16); v[3] = __uint_as_float(r.y & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(bf16* p, const float* v) {
+  bf16 b[4] = {from_f32<bf16>(v[0]), from_f32<bf16>(v[1]), from_f32<bf16>(v[2]), from_f32<bf16>(v[3])};
+  *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(b);
+}
+
 #define ACT_NONE 0
 #define ACT_SILU 1
 #define ACT_SIGMOID 2
@@ -146,24 +164,44 @@ __global__ __launch_bounds__(256) void decay_chunk_kernel(const T* __restrict__ 
     const int d = 32 * w + 8 * (i / 4) + 4 * half + i % 4;
     S[i] = (resume && e_live && d < D) ? kept[(size_t)d * E + e0 + col] : 0.f;
   }
+  // A chunk's inputs are asked for a chunk ahead and wait in registers as they were projected, so that the loads
+  // run under the products of the chunk before.
+  constexpr int QK_EACH = CHUNK * CHUNK_DP / 256, V_EACH = CHUNK * CHUNK / 256;
+  T q_next[QK_EACH], k_next[QK_EACH], v_next[V_EACH];
+  auto fetch = [&](int c0) {
+    const int n = min(CHUNK, len - c0);
+#pragma unroll
+    for (int it = 0; it < QK_EACH; ++it) {
+      const int idx = tid + 256 * it, t = idx / CHUNK_DP, d = idx % CHUNK_DP;
+      const bool in = t < n && d < D;
+      const T* row = proj + (size_t)(first + c0 + (in ? t : 0)) * ld + h * D + (in ? d : 0);
+      q_next[it] = in ? row[q_off] : from_f32<T>(0.f);
+      k_next[it] = in ? row[k_off] : from_f32<T>(0.f);
+    }
+#pragma unroll
+    for (int it = 0; it < V_EACH; ++it) {
+      const int idx = tid + 256 * it, t = idx / CHUNK, e = idx % CHUNK;
+      const bool in = t < n && e0 + e < E;
+      v_next[it] = in ? proj[(size_t)(first + c0 + t) * ld + v_off + h * E + e0 + e] : from_f32<T>(0.f);
+    }
+  };
+  if (len > 0) fetch(0);
   for (int c0 = 0; c0 < len; c0 += CHUNK) {
     const int n = min(CHUNK, len - c0);
     __syncthreads();  // the chunk before has been read (and pw written)
-    for (int idx = tid; idx < CHUNK * CHUNK_DP; idx += 256) {
-      const int t = idx / CHUNK_DP, d = idx % CHUNK_DP;
-      float qv = 0.f, kv = 0.f;
-      if (t < n && d < D) {
-        const T* row = proj + (size_t)(first + c0 + t) * ld;
-        qv = apply_act(to_f32(row[q_off + h * D + d]), act);
-        kv = apply_act(to_f32(row[k_off + h * D + d]), act) * k_scale;
-      }
-      Qs[t][d] = qv;
-      Ks[t][d] = kv;
+#pragma unroll
+    for (int it = 0; it < QK_EACH; ++it) {
+      const int idx = tid + 256 * it, t = idx / CHUNK_DP, d = idx % CHUNK_DP;
+      const bool in = t < n && d < D;
+      Qs[t][d] = in ? apply_act(to_f32(q_next[it]), act) : 0.f;
+      Ks[t][d] = in ? apply_act(to_f32(k_next[it]), act) * k_scale : 0.f;
     }
-    for (int idx = tid; idx < CHUNK * CHUNK; idx += 256) {
-      const int t = idx / CHUNK, e = idx % CHUNK;
-      Vs[t][e] = (t < n && e0 + e < E) ? apply_act(to_f32(proj[(size_t)(first + c0 + t) * ld + v_off + h * E + e0 + e]), act) : 0.f;
+#pragma unroll
+    for (int it = 0; it < V_EACH; ++it) {
+      const int idx = tid + 256 * it, t = idx / CHUNK, e = idx % CHUNK;
+      Vs[t][e] = (t < n && e0 + e < E) ? apply_act(to_f32(v_next[it]), act) : 0.f;
     }
+    if (c0 + CHUNK < len) fetch(c0 + CHUNK);
     __syncthreads();
     // A = Q K^T over this wave's 32 coordinates
     floatx16 acc;
@@ -255,22 +293,58 @@ __global__ __launch_bounds__(256) void decay_finish_kernel(const float* __restri
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
   const float* row = o + (size_t)t * n;
   const int gs = n / groups;
+  const bool by_four = gs % 4 == 0 && ld % 4 == 0 && g_off % 4 == 0;  // every row and group starts on 16 (8) bytes
   if (groups == 1) {
     __shared__ float red[17];
     float ss = 0.f;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) ss = fmaf(row[i], row[i], ss);
+    if (by_four) {
+      for (int i = 4 * threadIdx.x; i < n; i += 4 * blockDim.x) {
+        float v[4];
+        load4(row + i, v);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) ss = fmaf(v[c], v[c], ss);
+      }
+    } else {
+      for (int i = threadIdx.x; i < n; i += blockDim.x) ss = fmaf(row[i], row[i], ss);
+    }
     ss = block_sum(ss, red);
     if (threadIdx.x == 0) inv[0] = 1.0f / sqrtf(ss / (float)n + eps);
   } else {
     for (int g = wave; g < groups; g += waves) {
       float ss = 0.f;
-      for (int i = lane; i < gs; i += WAVE) ss = fmaf(row[g * gs + i], row[g * gs + i], ss);
+      if (by_four) {
+        for (int i = 4 * lane; i < gs; i += 4 * WAVE) {
+          float v[4];
+          load4(row + g * gs + i, v);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) ss = fmaf(v[c], v[c], ss);
+        }
+      } else {
+        for (int i = lane; i < gs; i += WAVE) ss = fmaf(row[g * gs + i], row[g * gs + i], ss);
+      }
       ss = wave_sum(ss);
       if (lane == 0) inv[g] = 1.0f / sqrtf(ss / (float)gs + eps);
     }
   }
   __syncthreads();
   const T* gate = proj + (size_t)t * ld + g_off;
+  if (by_four) {
+    for (int i = 4 * threadIdx.x; i < n; i += 4 * blockDim.x) {
+      float v[4], gt[4], gn[4] = {1.f, 1.f, 1.f, 1.f};
+      load4(row + i, v);
+      load4(gate + i, gt);
+      if (gain) load4(gain + i, gn);
+      const float scale = inv[i / gs];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        float r = v[c] * scale;
+        if (gain) r *= gn[c];
+        v[c] = r * apply_act(gt[c], gate_act);
+      }
+      store4(out + (size_t)t * n + i, v);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
     float v = row[i] * inv[i / gs];
     if (gain) v *= gain[i];

@@ -449,21 +449,23 @@ def test_linear_attention_keeps_a_far_key_and_forgets_by_its_decay():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_linear_attention_output_norm_and_gate(dtype):
+@pytest.mark.parametrize("sizes", [(3, 40, 5), (3, 40, 8), (2, 7, 4), (32, 128, 64)])
+def test_linear_attention_output_norm_and_gate(sizes, dtype):
+    """Rows and groups that start on 16 bytes (four values a load) and others."""
     from atomserve_amd.kernels import ops
 
-    T, H, E = 11, 3, 40
+    T, (H, E, off) = 11, sizes
     gen = torch.Generator().manual_seed(2)
     o = torch.randn(T, H, E, generator=gen) * 4
-    proj = bf(torch.randn(T, 5 + H * E, generator=gen))
+    proj = bf(torch.randn(T, off + H * E, generator=gen))
     gain = bf(1 + 0.1 * torch.randn(H * E, generator=gen))
     tol = 3e-6 if dtype == "float32" else 1e-2
     out = torch.empty((T, H * E), dtype=DTYPES[dtype], device=DEV)
-    ops.decay_finish(dev(o).view(T, H * E), H, 1e-5, None, dev(proj, DTYPES[dtype]), 5, "silu", out)
-    want = plain.rms(o.double(), 1e-5).reshape(T, -1) * torch.nn.functional.silu(proj[:, 5:].double())
+    ops.decay_finish(dev(o).view(T, H * E), H, 1e-5, None, dev(proj, DTYPES[dtype]), off, "silu", out)
+    want = plain.rms(o.double(), 1e-5).reshape(T, -1) * torch.nn.functional.silu(proj[:, off:].double())
     assert (out.float().cpu() - want).abs().max() <= tol * float(want.abs().max())
-    ops.decay_finish(dev(o).view(T, H * E), 1, 1e-5, dev(gain), dev(proj, DTYPES[dtype]), 5, "sigmoid", out)
-    want = plain.rms(o.double().reshape(T, -1), 1e-5) * gain.double() * torch.sigmoid(proj[:, 5:].double())
+    ops.decay_finish(dev(o).view(T, H * E), 1, 1e-5, dev(gain), dev(proj, DTYPES[dtype]), off, "sigmoid", out)
+    want = plain.rms(o.double().reshape(T, -1), 1e-5) * gain.double() * torch.sigmoid(proj[:, off:].double())
     assert (out.float().cpu() - want).abs().max() <= tol * float(want.abs().max())
 
 
