@@ -7,6 +7,7 @@
 // slot holds, a later row goes on from what the row before left.  Everything after the products is fp32.
 //
 //   decay_scan    token by token: a lane keeps a slice of one column of the state in registers for all of a row's tokens
+//   decay_step    a step of single tokens: the state read and written in whole lines (keys of up to 128, values in fours)
 //   decay_chunks  32 tokens at a time as four fp32 products on the matrix cores (keys of up to 128 coordinates)
 //   decay_finish  o normed in groups (per head, or all heads together) with an optional gain, times act(gate)
 #include "common.h"
@@ -116,6 +117,83 @@ extern "C" int as_decay_scan(const void* proj, int dtype, int ld, int q_off, int
   else if (dtype == DT_BF16)
     decay_scan_kernel<bf16><<<grid, 64, 0, stream>>>((const bf16*)proj, ld, q_off, k_off, v_off, H, D, E, act, k_scale, decay,
                                                      state, row_first, row_len, row_start, row_slots, out, SL, writes);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// ---- one token a row (a decode step) ------------------------------------------------------------------------
+// A step of single tokens is the state read once and written once: the wave's loads are whole 128-byte lines.  A
+// lane owns four neighbouring columns e of sixteen rows d of one head's state (eight lanes a line of 32 columns,
+// eight slices of d, whose partial sums meet by lane swaps).  Needs D <= 128 and E % 4 == 0.
+#define STEP_DPER 16
+
+template <typename T>
+__global__ __launch_bounds__(64) void decay_step_kernel(const T* __restrict__ proj, int ld, int q_off, int k_off,
+                                                        int v_off, int H, int D, int E, int act, float k_scale,
+                                                        const float* __restrict__ decay, float* __restrict__ state,
+                                                        const int* __restrict__ row_first,
+                                                        const int* __restrict__ row_start,
+                                                        const int* __restrict__ row_slots, float* __restrict__ out,
+                                                        int writes) {
+  const int lane = threadIdx.x, quad = lane & 7, sl = lane >> 3;
+  const int e = blockIdx.x * 32 + 4 * quad, h = blockIdx.y, r = blockIdx.z;
+  const bool live = e < E;  // E % 4 == 0: a lane's four columns are all there or none
+  const int t = row_first[r], slot = row_slots[r];
+  const float lam = decay[h];
+  const int d0 = sl * STEP_DPER;
+  float* kept = slot >= 0 ? state + (((size_t)slot * H + h) * D) * E : nullptr;
+  const bool resume = kept && row_start[r] > 0;
+  float S[STEP_DPER][4];
+#pragma unroll
+  for (int i = 0; i < STEP_DPER; ++i) {
+    if (resume && live && d0 + i < D) load4(kept + (size_t)(d0 + i) * E + e, S[i]);
+    else S[i][0] = S[i][1] = S[i][2] = S[i][3] = 0.f;
+  }
+  const T* row = proj + (size_t)t * ld;
+  float q[STEP_DPER], k[STEP_DPER], v[4];
+#pragma unroll
+  for (int i = 0; i < STEP_DPER; ++i) {
+    const bool in = d0 + i < D;
+    q[i] = in ? to_f32(row[q_off + h * D + d0 + i]) : 0.f;
+    k[i] = in ? to_f32(row[k_off + h * D + d0 + i]) : 0.f;
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) v[c] = live ? apply_act(to_f32(row[v_off + h * E + e + c]), act) : 0.f;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < STEP_DPER; ++i) {
+    const float qa = apply_act(q[i], act), ka = apply_act(k[i], act) * k_scale;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      S[i][c] = fmaf(lam, S[i][c], ka * v[c]);
+      acc[c] = fmaf(S[i][c], qa, acc[c]);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+    for (int off = 8; off < WAVE; off <<= 1) acc[c] += __shfl_xor(acc[c], off, WAVE);
+  if (live && sl == 0) store4(out + ((size_t)t * H + h) * E + e, acc);
+  if (kept && writes && live) {
+#pragma unroll
+    for (int i = 0; i < STEP_DPER; ++i)
+      if (d0 + i < D) store4(kept + (size_t)(d0 + i) * E + e, S[i]);
+  }
+}
+
+extern "C" int as_decay_step(const void* proj, int dtype, int ld, int q_off, int k_off, int v_off, int H, int D, int E,
+                             int act, float k_scale, const float* decay, float* state, const int* row_first,
+                             const int* row_start, const int* row_slots, int num_rows, float* out, int writes,
+                             hipStream_t stream) {
+  if (num_rows <= 0) return AS_OK;
+  if (H <= 0 || D <= 0 || E <= 0 || D > 8 * STEP_DPER || E % 4 || act < 0 || act > 2) return AS_BAD_SHAPE;
+  dim3 grid((E + 31) / 32, H, num_rows);
+  if (grid.y > 65535 || grid.z > 65535) return AS_BAD_SHAPE;
+  if (dtype == DT_F32)
+    decay_step_kernel<float><<<grid, 64, 0, stream>>>((const float*)proj, ld, q_off, k_off, v_off, H, D, E, act, k_scale, decay,
+                                                      state, row_first, row_start, row_slots, out, writes);
+  else if (dtype == DT_BF16)
+    decay_step_kernel<bf16><<<grid, 64, 0, stream>>>((const bf16*)proj, ld, q_off, k_off, v_off, H, D, E, act, k_scale, decay,
+                                                     state, row_first, row_start, row_slots, out, writes);
   else return AS_BAD_DTYPE;
   return launch_status();
 }

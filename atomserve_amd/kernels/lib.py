@@ -46,6 +46,7 @@ SIGNATURES = {
     "as_clamped_gate": ("layer_ops", [P, P, I, I, I, F, F, P]),
     "as_decay_scan": ("linear_attention", [P, I, I, I, I, I, I, I, I, I, F, P, P, P, P, P, P, I, P, I, P]),
     "as_decay_chunks": ("linear_attention", [P, I, I, I, I, I, I, I, I, I, F, P, P, P, P, P, P, I, P, I, P]),
+    "as_decay_step": ("linear_attention", [P, I, I, I, I, I, I, I, I, I, F, P, P, P, P, P, I, P, I, P]),
     "as_decay_finish": ("linear_attention", [P, I, I, F, P, P, I, I, I, I, P, I, P]),
     "as_rows_rms_norm": ("latent", [P, I, I, I, I, P, F, P, I, P]),
     "as_latent_kv_store": ("latent", [P, I, I, I, I, I, P, F, P, P, P, P, I, I, I, P]),

@@ -1669,11 +1669,38 @@ def decay_chunks(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_
          _ptr(out), int(bool(writes)), _stream())  # fmt: skip
 
 
+def decay_step(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out,
+               writes=True) -> None:  # fmt: skip
+    """What `decay_scan` computes for a step in which every row is ONE token (only each row's first token is taken):
+    the state is read and written once, in whole lines.  Keys of up to DECAY_CHUNKS_MAX_DIM, values a multiple of 4."""
+    _check(proj, "proj", (F32, BF16), (None, None))
+    T, ld = proj.shape
+    H, D, E = num_heads, dim, vdim
+    if activation not in (None, "silu"):
+        raise KernelError(f"decay_step: activation {activation!r} (None or 'silu')")
+    if min(H, D, E) < 1 or D > DECAY_CHUNKS_MAX_DIM or E % 4 or max(q_off + H * D, k_off + H * D, v_off + H * E) > ld or min(q_off, k_off, v_off) < 0:
+        raise KernelError(f"decay_step: {H} heads of {D} and {E} at columns {q_off}, {k_off}, {v_off} of {ld}")
+    _check(decay, "decay", F32, (H,))
+    _check(state, "state", F32, (None, H, D, E))
+    _check(out, "out", F32, (T, H, E))
+    R = _check_rows(step_rows, T)
+    _, row_first, row_len, row_start, row_slots = step_rows
+    call("as_decay_step", _ptr(proj), _DT[proj.dtype], ld, q_off, k_off, v_off, H, D, E, ACTIVATIONS[activation],
+         float(k_scale), _ptr(decay), _ptr(state), _ptr(row_first), _ptr(row_start), _ptr(row_slots), R, _ptr(out),
+         int(bool(writes)), _stream())  # fmt: skip
+
+
 def decay_attention(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out,
                     writes=True) -> None:  # fmt: skip
     """What `decay_scan` computes, by whichever kernel suits the step: token by token where every row is one token (a
-    decode step: step_rows names no row per token) or the keys are wider than the chunked kernel takes, else in chunks."""
-    kernel = decay_scan if step_rows[0] is None or dim > DECAY_CHUNKS_MAX_DIM else decay_chunks
+    decode step: step_rows names no row per token; values in fours through the kernel that moves whole lines) or the keys
+    are wider than the chunked kernel takes, else in chunks."""
+    if dim > DECAY_CHUNKS_MAX_DIM:
+        kernel = decay_scan
+    elif step_rows[0] is None:
+        kernel = decay_step if vdim % 4 == 0 else decay_scan
+    else:
+        kernel = decay_chunks
     kernel(proj, q_off, k_off, v_off, num_heads, dim, vdim, activation, k_scale, decay, state, step_rows, out, writes)
 
 

@@ -385,7 +385,7 @@ def test_average_over_the_layers_results(dtype):
 
 def run_decay(q, k, v, decay, act, k_scale, cuts, dtype, slot=1, state=None, kernel=None):
     """The scan over one request cut into rows of `cuts` tokens (one call each), q, k, v given before the activation.
-    kernel: "decay_scan" or "decay_chunks" to name one; None: as a step would choose (single tokens as a decode step)."""
+    kernel: "decay_scan", "decay_chunks" or (single tokens) "decay_step" to name one; None: as a step would choose (single tokens as a decode step)."""
     from atomserve_amd.kernels import ops
 
     T, H, D = q.shape
@@ -423,7 +423,10 @@ def test_linear_attention_with_decays(shape, dtype):
         want = plain.decayed_state_scan(f(q), f(k) * k_scale, f(v), decay).float()
         tol = 2e-5 * float(want.abs().max())
         kernels = ("decay_scan", "decay_chunks") if D <= 128 else ("decay_scan",)
-        for cuts, kernel in [(c, kn) for c in ([T], [1] * T, [2, 31, 1, 1, 30, 2], [32, 33, 2]) for kn in kernels] + [([1] * T, None), ([T], None)]:
+        ways = [(c, kn) for c in ([T], [1] * T, [2, 31, 1, 1, 30, 2], [32, 33, 2]) for kn in kernels] + [([1] * T, None), ([T], None)]
+        if D <= 128 and E % 4 == 0:
+            ways.append(([1] * T, "decay_step"))
+        for cuts, kernel in ways:
             got, state = run_decay(q, k, v, decay, act, k_scale, cuts, dtype, kernel=kernel)
             assert (got - want).abs().max() <= tol, f"{shape} {act} {cuts} {kernel}: {float((got - want).abs().max()):.3e} of {float(want.abs().max()):.3e}"
         assert bool((state[0] == 5.0).all()) and bool((state[2] == 5.0).all())  # the other slots are not touched
