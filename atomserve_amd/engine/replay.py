@@ -151,7 +151,7 @@ def build_parser() -> argparse.ArgumentParser:
                    help="most tokens that live requests hold at any time, each request's count rounded up to 64")  # fmt: skip
     p.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     p.add_argument("--pages", type=int, default=None, help="pages in the cache pool (default: what --max-tokens needs)")
-    p.add_argument("--max-live", type=int, default=8, help="most requests alive at once")
+    p.add_argument("--max-live", type=int, default=4, help="most requests alive at once: the number of state slots")
     p.add_argument("--timed-products", action="store_true",
                    help="let the library's matrix products be chosen by timing, as in serving")  # fmt: skip
     p.add_argument("--device", default="cuda:0", help=argparse.SUPPRESS)
