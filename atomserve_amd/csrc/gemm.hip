@@ -162,6 +162,8 @@ struct NormLink {
   const float* gain;    // LINK: [N], the gains of the norm that follows
   bf16* scaled;         // LINK: [M, N]
   float* ssq_out;       // LINK: [M, strips of this product]
+  float limit;          // GATED: 0: silu(gate) * up; > 0: g sigmoid(alpha g) (u + 1), g = min(gate, limit), u = clamp(up, +-limit)
+  float alpha;
 };
 
 // The LINK epilogue for the lane that holds columns n .. n+3 of row m (sum: the product's fp32
@@ -464,8 +466,13 @@ __global__ __launch_bounds__(PIPE_WAVES * 64) void gemm_bf16_skinny_pipe_kernel(
           if (GATED) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const float g = rounded<OutT>(gate[mt][r]);
-              sum[r] = g / (1.0f + expf(-g)) * rounded<OutT>(sum[r]);
+              const float g = rounded<OutT>(gate[mt][r]), u = rounded<OutT>(sum[r]);
+              if (link.limit > 0.f) {
+                const float gl = fminf(g, link.limit), ul = fminf(fmaxf(u, -link.limit), link.limit);
+                sum[r] = gl / (1.0f + expf(-link.alpha * gl)) * (ul + 1.0f);
+              } else {
+                sum[r] = g / (1.0f + expf(-g)) * u;
+              }
             }
           }
           if (m < M && n < N) store4<OutT>(out + (size_t)m * N + n, sum, min(4, N - n));
@@ -549,6 +556,18 @@ extern "C" int as_gemm_bf16_gated(const void* a, const void* w, const void* wt, 
   if (M <= 0) return AS_OK;
   if (N <= 0 || K <= 0 || (K & 7) || !pipe_fits(M, K)) return AS_BAD_SHAPE;
   return dispatch_pipe<true, bf16>(a, w, wt, out, M, N, K, stream);
+}
+
+// The same with the gated activation with limits: g = min(gate, limit), u = clamp(up, -limit, limit),
+// out = g sigmoid(alpha g) (u + 1), both products rounded to bf16 first.
+extern "C" int as_gemm_bf16_gated_limited(const void* a, const void* w, const void* wt, void* out, int M, int N, int K,
+                                          float limit, float alpha, hipStream_t stream) {
+  if (M <= 0) return AS_OK;
+  if (N <= 0 || K <= 0 || (K & 7) || !pipe_fits(M, K) || !(limit > 0.f)) return AS_BAD_SHAPE;
+  NormLink link = {};
+  link.limit = limit;
+  link.alpha = alpha;
+  return dispatch_pipe<true, bf16>(a, w, wt, out, M, N, K, stream, link);
 }
 
 // The producer of a NormLink: x[M, N] (fp32) += bf16(a @ w^T); scaled[M, N] = bf16(x * gain);

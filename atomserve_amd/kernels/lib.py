@@ -63,6 +63,7 @@ SIGNATURES = {
     "as_gemm_f32": ("gemm", [P, P, P, I, I, I, P]),
     "as_gemm_bf16_skinny": ("gemm", [P, P, P, P, I, I, I, I, I, P]),
     "as_gemm_bf16_gated": ("gemm", [P, P, P, P, I, I, I, P]),
+    "as_gemm_bf16_gated_limited": ("gemm", [P, P, P, P, I, I, I, F, F, P]),
     "as_gemm_bf16_link": ("gemm", [P, P, P, P, P, P, P, I, I, I, P]),
     "as_gemm_bf16_scaled": ("gemm", [P, P, I, F, P, P, P, I, I, I, I, P]),
     "as_wave_order": ("gemm", [P, P, I, I, P]),

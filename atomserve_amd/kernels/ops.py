@@ -1611,7 +1611,17 @@ def clamped_gate(gate_up, out, limit: float) -> None:
 
 def gemm_clamped_gate(a, w, out, limit: float, choices=None) -> None:
     """out = clamped_gate(a @ w^T, limit): w [2 I, K] holds the gate rows, then the up rows; out [T, I]."""
-    gate_up = torch.empty((a.shape[0], _rows(w).shape[0]), dtype=a.dtype, device=a.device)
+    M, K = a.shape
+    rows = _rows(w)
+    inter = rows.shape[0] // 2
+    if a.dtype == BF16 and M and limit > 0 and (_few_rows(M, K, inter, GATED_MAX_K, w=w) or _gated_two_tiles(M, K, w)):
+        # few rows: the product that streams the weights applies the activation on its way out
+        _check(rows, "w", a.dtype, (2 * inter, K))
+        _check(out, "out", a.dtype, (M, inter))
+        call("as_gemm_bf16_gated_limited", _ptr(a), _ptr(rows), _wave_ptr(w), _ptr(out), M, inter, K, float(limit),
+             CLAMPED_GATE_ALPHA, _stream())  # fmt: skip
+        return
+    gate_up = torch.empty((M, rows.shape[0]), dtype=a.dtype, device=a.device)
     gemm(a, w, gate_up, choices)
     clamped_gate(gate_up, out, limit)
 

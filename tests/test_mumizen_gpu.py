@@ -680,6 +680,27 @@ def test_gated_activation_with_limits(limit, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rows", [1, 8, 24, 70])
+def test_gated_product_with_limits(rows, dtype):
+    """The product [gate | up] with the activation: few bfloat16 rows through the kernel that applies it on its way
+    out, the others through the product and the activation's own kernel; both round the two products first."""
+    from atomserve_amd.kernels import ops
+
+    K, inner, limit = 256, 96, 1.25
+    gen = torch.Generator().manual_seed(rows)
+    a, w = bf(torch.randn(rows, K, generator=gen)), bf(0.2 * torch.randn(2 * inner, K, generator=gen))
+    t = DTYPES[dtype]
+    out = torch.empty((rows, inner), dtype=t, device=DEV)
+    for weights in (dev(w, t), ops.Streamed(dev(w, t), True)):
+        ops.gemm_clamped_gate(dev(a, t), weights, out, limit, ops.ProductChoices(fixed=True))
+        prod = a.double() @ w.double().t()
+        if dtype == "bfloat16":
+            prod = bf(prod.float()).double()
+        want = plain.clamped_gate(prod[:, :inner], prod[:, inner:], limit)
+        assert (out.float().cpu() - want).abs().max() <= (3e-6 if dtype == "float32" else 1e-2) * float(want.abs().max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("sizes", [(5, 2, 40, 24), (7, 1, 24, 0), (3, 3, 16, 16), (70, 9, 8, 8), (2, 2, 264, 0)])
 def test_gated_routed_experts_alone(sizes, dtype):
     """The router's choice (logits with a bias, the largest) and weights (softmax over the chosen) against the plain
