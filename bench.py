@@ -215,7 +215,7 @@ def mumizen_config(width: int, layers: int, vocab: int):
 
     heads = width // 128
     decay = {"heads": heads, "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** -(5.0 + 5.0 * h / heads) for h in range(heads)]}
-    rot = {"dims": 64, "base": 1e6, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    rot = {"dims": 64, "base": 1e6, "scaling": {"factor": 16.0, "original": 4096, "fast": 16.0, "slow": 2.0}}
     latent = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": width // 2, "kv_rank": 192,
               "scale": 192**-0.5, "rot": rot}  # fmt: skip
     dense = {"kind": "dense", "ff": 3 * width, "limit": 7.0}

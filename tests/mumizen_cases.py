@@ -60,9 +60,9 @@ CASES = {
     "latents": {
         "architecture": "Mumizen", "vocab": 300, "width": 128, "norm": {"eps": 1e-5, "groups": 4},
         "layers": [
-            {"type": "latent_attention", "mixer": _latent(4, 32, 32, 32, 48, 128, 0.125, 250000.0, (16.0, 32, 8.0, 1.0)), "mlp": _dense(64, 0.875)},
-            {"type": "latent_attention", "mixer": _latent(8, 8, 32, 24, 32, 128, 0.18, 250000.0, (16.0, 32, 8.0, 1.0), kv_from=0), "mlp": _moe(32, 2.0, 9, 4, (8, 1.5))},
-            {"type": "latent_attention", "mixer": _latent(2, 40, 32, 16, 64, 128, 0.11, 250000.0, (16.0, 32, 8.0, 1.0), kv_from=0), "mlp": None},
+            {"type": "latent_attention", "mixer": _latent(4, 32, 32, 32, 48, 128, 0.125, 300000.0, (16.0, 32, 8.0, 1.0)), "mlp": _dense(64, 0.875)},
+            {"type": "latent_attention", "mixer": _latent(8, 8, 32, 24, 32, 128, 0.18, 300000.0, (16.0, 32, 8.0, 1.0), kv_from=0), "mlp": _moe(32, 2.0, 9, 4, (8, 1.5))},
+            {"type": "latent_attention", "mixer": _latent(2, 40, 32, 16, 64, 128, 0.11, 300000.0, (16.0, 32, 8.0, 1.0), kv_from=0), "mlp": None},
             {"type": "latent_attention", "mixer": _latent(6, 16, 2, 8, 8, 56, 0.25, 7.0, (2.0, 16, 4.0, 0.5)), "mlp": _dense(24, 6.0)},
         ],
     },  # fmt: skip
@@ -79,9 +79,9 @@ CASES = {
         "architecture": "Mumizen", "vocab": 203, "width": 88, "norm": {"eps": 1e-6, "groups": 2},
         "layers": [
             {"type": "retention", "mixer": _decay(3, 10, 14, (0.99, 0.9, 0.75)), "mlp": _dense(20, 1.0)},
-            {"type": "latent_attention", "mixer": _latent(3, 10, 6, 10, 20, 36, 0.25, 1000.0, (8.0, 32, 32.0, 1.0)), "mlp": _moe(12, 1.5, 6, 3, (20, 2.0))},
-            {"type": "lightning", "mixer": _decay(5, 6, 6, (0.6, 0.8, 0.9, 0.97, 0.999)), "mlp": _moe(12, 1.5, 4, 2)},
-            {"type": "latent_attention", "mixer": _latent(7, 6, 6, 10, 12, 36, 0.3, 1000.0, (8.0, 32, 32.0, 1.0), kv_from=1), "mlp": _dense(28, 2.0)},
+            {"type": "latent_attention", "mixer": _latent(3, 10, 6, 10, 20, 36, 0.25, 1000.0, (6.0, 32, 24.0, 1.5)), "mlp": _moe(12, 1.75, 6, 3, (20, 2.25))},
+            {"type": "lightning", "mixer": _decay(5, 6, 6, (0.55, 0.7, 0.85, 0.95, 0.998)), "mlp": _moe(12, 1.75, 4, 2)},
+            {"type": "latent_attention", "mixer": _latent(7, 6, 6, 10, 12, 36, 0.3, 1000.0, (6.0, 32, 24.0, 1.5), kv_from=1), "mlp": _dense(28, 2.0)},
         ],
     },  # fmt: skip
 }

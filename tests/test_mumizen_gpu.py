@@ -483,7 +483,7 @@ def test_scaled_rotation_table():
         num_tokens = 9
 
     env = BuildEnv(torch.float32, torch.device(DEV))
-    for dims, base, scaling in ((16, 250000.0, (8.0, 512, 32.0, 1.0)), (6, 50.0, (3.0, 20, 4.0, 0.5)), (64, 10000.0, (40.0, 4096, 32.0, 1.0)),
+    for dims, base, scaling in ((16, 200000.0, (6.0, 256, 24.0, 1.5)), (6, 50.0, (3.0, 20, 4.0, 0.5)), (64, 10000.0, (40.0, 4096, 16.0, 2.0)),
                                 (2, 7.0, (2.0, 16, 4.0, 0.5)), (8, 100.0, None)):  # fmt: skip
         rot = {"dims": dims, "base": base}
         if scaling:
