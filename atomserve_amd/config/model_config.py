@@ -5,7 +5,7 @@ number of its own.  Field meanings and the rejected options follow the reference
 (atomserve/config.py:15-65).
 """
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 
 
 class ConfigError(ValueError):
@@ -646,3 +646,251 @@ class MumizenConfig:
                   for layer in self.layers]  # fmt: skip
         return {"architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
                 "norm": {"eps": self.norm_eps, "groups": self.norm_groups}, "layers": layers}  # fmt: skip
+
+
+# ---- Natatar ------------------------------------------------------------------------------------------
+
+
+def _rotation(raw, where: str):
+    """(dims, base, scaling) of a mixer's `rot`, scaling None or (factor, original, fast, slow); None without `rot`."""
+    if not raw:
+        return None
+    scaling = raw.get("scaling")
+    if scaling:
+        scaling = tuple(float(_need(scaling, k, where + "scaling.")) for k in ("factor", "original", "fast", "slow"))
+    return (int(_need(raw, "dims", where)), float(_need(raw, "base", where)), scaling or None)
+
+
+def _rotation_dict(rot) -> dict:
+    raw = {"dims": rot[0], "base": rot[1]}
+    if rot[2]:
+        raw["scaling"] = dict(zip(("factor", "original", "fast", "slow"), rot[2]))
+    return raw
+
+
+@dataclass(frozen=True)
+class NatatarAttention:
+    """A softmax attention's sizes and options.  As a layer's own mixer ("attention") it has biases, a norm over the
+    whole of q and of k and, with v_mix, values mixed with those of the first such layer; as the left half of a
+    "parallel" mixer it has a rotation and an output gate instead."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    v_mix: bool = False
+    rot: object = None  # None, or (dims, base, scaling)
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "NatatarAttention":
+        return cls(*(int(_need(raw, k, where)) for k in ("heads", "kv_heads", "dim", "vdim")),
+                   scale=float(_need(raw, "scale", where)), v_mix=bool(raw.get("v_mix", False)),
+                   rot=_rotation(raw.get("rot"), where + "rot."))  # fmt: skip
+
+    def to_dict(self) -> dict:
+        raw = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale}
+        if self.v_mix:
+            raw["v_mix"] = True
+        if self.rot:
+            raw["rot"] = _rotation_dict(self.rot)
+        return raw
+
+
+@dataclass(frozen=True)
+class NatatarMemory:
+    """A matrix memory with exponential gates (the right half of a "parallel" mixer)."""
+
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "NatatarMemory":
+        return cls(*(int(_need(raw, k, where)) for k in ("heads", "dim", "vdim")), gate_cap=float(_need(raw, "gate_cap", where)))
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "dim": self.dim, "vdim": self.vdim, "gate_cap": self.gate_cap}
+
+
+@dataclass(frozen=True)
+class NatatarParallel:
+    left: NatatarAttention
+    right: NatatarMemory
+    left_scale: float
+    right_scale: float
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "NatatarParallel":
+        return cls(NatatarAttention.from_dict(_need(raw, "left", where), where + "left."),
+                   NatatarMemory.from_dict(_need(raw, "right", where), where + "right."),
+                   float(_need(raw, "left_scale", where)), float(_need(raw, "right_scale", where)))  # fmt: skip
+
+    def to_dict(self) -> dict:
+        return {"left": self.left.to_dict(), "right": self.right.to_dict(), "left_scale": self.left_scale,
+                "right_scale": self.right_scale}  # fmt: skip
+
+
+@dataclass(frozen=True)
+class NatatarChannelDelta:
+    """A gated delta rule with a decay per head and key channel.  The ranks of the two-step projections (of the
+    decay's step size and of the output gate) are sizes that only the checkpoint's shapes tell: a configuration
+    read from a model folder is completed from them, one written by this package names them itself."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    decay_rank: int = 0
+    gate_rank: int = 0
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "NatatarChannelDelta":
+        return cls(*(int(_need(raw, k, where)) for k in ("heads", "kv_heads", "dim", "vdim", "conv")),
+                   decay_rank=int(raw.get("decay_rank", 0)), gate_rank=int(raw.get("gate_rank", 0)))  # fmt: skip
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "conv": self.conv,
+                "decay_rank": self.decay_rank, "gate_rank": self.gate_rank}  # fmt: skip
+
+
+@dataclass(frozen=True)
+class NatatarExperts:
+    ff: int
+    experts: int
+    top: int
+    scale: float = 1.0
+    groups: int = 1  # equal groups of neighbouring experts
+    keep: int = 1  # groups of which experts can be chosen
+
+    @classmethod
+    def from_dict(cls, raw: dict, where: str) -> "NatatarExperts":
+        kind = _need(raw, "kind", where)
+        if kind != "moe":
+            raise ConfigError(f"{where}kind={kind!r} is not supported ('moe')")
+        expert, router = _need(raw, "expert", where), _need(raw, "router", where)
+        groups = router.get("groups") or {}
+        count = int(groups.get("count", 1))
+        return cls(int(_need(expert, "ff", where + "expert.")), int(_need(router, "experts", where + "router.")),
+                   int(_need(router, "top", where + "router.")), float(router.get("scale", 1.0)), count,
+                   int(groups.get("keep", count)))  # fmt: skip
+
+    def to_dict(self) -> dict:
+        router = {"experts": self.experts, "top": self.top, "scale": self.scale}
+        if self.groups > 1:
+            router["groups"] = {"count": self.groups, "keep": self.keep}
+        return {"kind": "moe", "expert": {"ff": self.ff}, "router": router}
+
+
+@dataclass(frozen=True)
+class NatatarLayer:
+    type: str  # "attention", "parallel" or "channel_delta"
+    mixer: object
+    mlp: object  # NatatarExperts or None
+
+
+@dataclass(frozen=True)
+class NatatarConfig:
+    """A Natatar decoder: pre-norm layers over several residual streams that every sublayer reads as one weighted
+    sum and writes back through a mixing matrix; norms whose gains are stored around zero; mixers of three kinds
+    (a biased softmax attention that may mix its values with an earlier layer's, a rotary gated attention beside a
+    matrix memory, a delta rule with decays per key channel); feed-forwards of experts chosen within the best
+    groups; the embedding table, scaled on the way in, is also the head."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: tuple  # of NatatarLayer
+    residual_mult: float = 1.0
+    embedding_scale: float = 1.0
+    streams: int = 0  # 0: one stream and plain residual sums
+
+    architecture = "Natatar"
+    MIXERS = ("attention", "parallel", "channel_delta")
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "NatatarConfig":
+        _require(raw, ["vocab", "width", "layers", "norm"])
+        layers = []
+        for i, entry in enumerate(raw["layers"]):
+            where = f"layers[{i}]."
+            kind = _need(entry, "type", where)
+            mixer = _need(entry, "mixer", where)
+            if kind == "attention":
+                mixer = NatatarAttention.from_dict(mixer, where + "mixer.")
+            elif kind == "parallel":
+                mixer = NatatarParallel.from_dict(mixer, where + "mixer.")
+            elif kind == "channel_delta":
+                mixer = NatatarChannelDelta.from_dict(mixer, where + "mixer.")
+            else:
+                raise ConfigError(f"{where}type={kind!r} is not supported (one of {', '.join(cls.MIXERS)})")
+            mlp = entry.get("mlp")
+            layers.append(NatatarLayer(kind, mixer, None if mlp is None else NatatarExperts.from_dict(mlp, where + "mlp.")))
+        cfg = cls(
+            vocab_size=int(raw["vocab"]),
+            hidden_size=int(raw["width"]),
+            norm_eps=float(_need(raw["norm"], "eps", "norm.")),
+            layers=tuple(layers),
+            residual_mult=float(raw.get("residual_mult", 1.0)),
+            embedding_scale=float((raw.get("embedding") or {}).get("scale", 1.0)),
+            streams=int(raw.get("streams") or 0),
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size < 1 or self.hidden_size < 1 or not self.layers:
+            raise ConfigError("vocab, width and the number of layers must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        if self.streams < 0:
+            raise ConfigError("streams is not negative")
+        mixed = None
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            for a in ([m] if layer.type == "attention" else [m.left] if layer.type == "parallel" else []):
+                if min(a.heads, a.kv_heads, a.dim, a.vdim) < 1 or a.heads % a.kv_heads:
+                    raise ConfigError(f"layers[{i}]: head counts and sizes must be positive, heads a multiple of kv_heads")
+                if a.rot and (a.rot[0] < 2 or a.rot[0] % 2 or a.rot[0] > a.dim or not a.rot[1] > 1):
+                    raise ConfigError(f"layers[{i}]: rot.dims is even and at most dim, rot.base exceeds 1")
+            if layer.type == "attention" and m.v_mix:
+                if mixed is not None and (mixed.kv_heads, mixed.vdim) != (m.kv_heads, m.vdim):
+                    raise ConfigError(f"layers[{i}]: layers that mix values have values of one shape")
+                mixed = mixed or m
+            if layer.type == "parallel" and min(m.right.heads, m.right.dim, m.right.vdim) < 1:
+                raise ConfigError(f"layers[{i}]: the memory's head count and sizes must be positive")
+            if layer.type == "parallel" and not m.right.gate_cap > 0:
+                raise ConfigError(f"layers[{i}]: gate_cap must be positive")
+            if layer.type == "channel_delta":
+                if min(m.heads, m.kv_heads, m.dim, m.vdim, m.conv) < 1 or m.heads % m.kv_heads:
+                    raise ConfigError(f"layers[{i}]: head counts and sizes must be positive, heads a multiple of kv_heads")
+            f = layer.mlp
+            if f is not None:
+                if f.ff < 1 or not 1 <= f.top <= f.experts:
+                    raise ConfigError(f"layers[{i}].mlp: sizes must be positive and top at most the number of experts")
+                if f.groups < 1 or f.experts % f.groups or not 1 <= f.keep <= f.groups or f.keep * (f.experts // f.groups) < f.top:
+                    raise ConfigError(f"layers[{i}].mlp: experts divide into equal groups, and the kept groups hold at least top experts")
+
+    def completed(self, shape_of) -> "NatatarConfig":
+        """This configuration with the sizes that only tensors tell: shape_of(checkpoint name) -> shape or None."""
+        layers = []
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            if layer.type == "channel_delta":
+                a1, g1 = shape_of(f"l{i}.mix.a1"), shape_of(f"l{i}.mix.g1")
+                m = replace(m, decay_rank=int(a1[0]) if a1 else m.decay_rank, gate_rank=int(g1[0]) if g1 else m.gate_rank)
+            layers.append(replace(layer, mixer=m))
+        return replace(self, layers=tuple(layers))
+
+    def to_dict(self) -> dict:
+        """The config.json that `from_dict` reads back to this object."""
+        layers = [{"type": layer.type, "mixer": layer.mixer.to_dict(), "mlp": None if layer.mlp is None else layer.mlp.to_dict()}
+                  for layer in self.layers]  # fmt: skip
+        raw = {"architecture": self.architecture, "vocab": self.vocab_size, "width": self.hidden_size,
+               "norm": {"eps": self.norm_eps}, "residual_mult": self.residual_mult,
+               "embedding": {"scale": self.embedding_scale}, "layers": layers}  # fmt: skip
+        if self.streams:
+            raw["streams"] = self.streams
+        return raw

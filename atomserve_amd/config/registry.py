@@ -25,6 +25,9 @@ class Architecture:
                     "log_rate" (small values around 0), "near_identity" (a square matrix around the
                     identity), "fraction" (values between 0 and 1), "depth_weights" (mostly on the last entry), "expert_table:<experts>" (int32 rows of distinct expert numbers)
     ignored:        typed configuration -> checkpoint names that may be present and unused
+    complete:       (typed configuration, shape_of) -> the configuration with the sizes that config.json leaves to
+                    the tensors' shapes (shape_of(checkpoint name) -> shape, or None for a name the folder lacks);
+                    None: config.json tells every size
     """
 
     name: str
@@ -33,6 +36,7 @@ class Architecture:
     checkpoint_map: Callable[[Any], dict]
     checkpoint_shapes: Callable[[Any], dict]
     ignored: Callable[[Any], set] = lambda config: set()
+    complete: Any = None
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}
@@ -72,7 +76,12 @@ def load_model_config(model_dir: str) -> tuple[Architecture, Any]:
     with open(path) as f:
         raw = json.load(f)
     arch = architecture_for(raw)
-    return arch, arch.parse_config(raw)
+    config = arch.parse_config(raw)
+    if arch.complete is not None:
+        from atomserve_amd.weights.loader import checkpoint_shapes_of
+
+        config = arch.complete(config, checkpoint_shapes_of(model_dir))
+    return arch, config
 
 
 def _load_builtin() -> None:
@@ -80,4 +89,5 @@ def _load_builtin() -> None:
     import atomserve_amd.models.dozusun  # noqa: F401
     import atomserve_amd.models.koravik  # noqa: F401
     import atomserve_amd.models.mumizen  # noqa: F401
+    import atomserve_amd.models.natatar  # noqa: F401
     import atomserve_amd.models.qwen3  # noqa: F401

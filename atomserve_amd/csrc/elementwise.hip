@@ -681,6 +681,104 @@ extern "C" int as_head_norm_store(const void* proj, int dtype, int ld, int q_off
   return launch_status();
 }
 
+// ---- heads out of a wider projection, normed over the whole projection ---------------------------------
+// As head_norm_store, with three more things a design may ask for.  Biases q_bias [H dim], k_bias [KV dim], v_bias
+// [KV vdim] (fp32, or none) are added to the projection's output first.  With gains qw [H dim] and kw [KV dim] (fp32)
+// queries and keys are RMS-normed over ALL their heads at once: x / sqrt(mean over H dim (x^2) + eps) * gain.  The
+// values may be mixed with those that an earlier layer kept for the same tokens: v_mode 1 writes this layer's values
+// (bias added) into v_keep fp32 [T, KV vdim]; v_mode 2 stores (1 - lam) v + lam v_keep[t] instead of v.  The rotation
+// (after the norm) and the layout of q_out and of the pages are head_norm_store's.  A workgroup per token.
+template <typename T>
+__global__ __launch_bounds__(256) void whole_norm_store_kernel(
+    const T* __restrict__ proj, int ld, int q_off, int k_off, int v_off, int H, int KV, int dim, int vdim, int Dp,
+    const float* __restrict__ q_bias, const float* __restrict__ k_bias, const float* __restrict__ v_bias,
+    const float* __restrict__ qw, const float* __restrict__ kw, float eps, const float2* __restrict__ cs, int R,
+    float* __restrict__ v_keep, int v_mode, float lam, const int* __restrict__ slots, T* __restrict__ q_out,
+    T* __restrict__ k_pages, T* __restrict__ v_pages, int bs, int store) {
+  __shared__ float red[17];
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * ld;
+  const int nq = H * dim, nk = KV * dim, nv = KV * vdim;
+  float inv_q = 1.f, inv_k = 1.f;
+  if (qw) {
+    float sq = 0.f, sk = 0.f;
+    for (int c = threadIdx.x; c < nq; c += blockDim.x) {
+      const float v = to_f32(row[q_off + c]) + (q_bias ? q_bias[c] : 0.f);
+      sq = fmaf(v, v, sq);
+    }
+    for (int c = threadIdx.x; c < nk; c += blockDim.x) {
+      const float v = to_f32(row[k_off + c]) + (k_bias ? k_bias[c] : 0.f);
+      sk = fmaf(v, v, sk);
+    }
+    inv_q = 1.0f / sqrtf(block_sum(sq, red) / (float)nq + eps);
+    inv_k = 1.0f / sqrtf(block_sum(sk, red) / (float)nk + eps);
+  }
+  const int half = cs ? R / 2 : 0;
+  const int slot = (store && slots) ? slots[t] : -1;
+  // queries, then keys: coordinate d of head hh, with its partner if it turns
+  for (int which = 0; which < 2; ++which) {
+    const int heads = which ? KV : H, off = which ? k_off : q_off;
+    const float* bias = which ? k_bias : q_bias;
+    const float* w = which ? kw : qw;
+    const float inv = which ? inv_k : inv_q;
+    if (which && slot < 0) break;
+    for (int idx = threadIdx.x; idx < heads * Dp; idx += blockDim.x) {
+      const int hh = idx / Dp, d = idx - hh * Dp;
+      auto value = [&](int dd) {
+        const int c = hh * dim + dd;
+        float v = to_f32(row[off + c]) + (bias ? bias[c] : 0.f);
+        if (w) v = v * inv * w[c];
+        return v;
+      };
+      float v = d < dim ? value(d) : 0.f;
+      if (d < 2 * half) {
+        const int i = d < half ? d : d - half, o = d < half ? d + half : d - half;
+        const float u = value(o);
+        const float2 a = cs[(size_t)t * half + i];
+        v = d < half ? v * a.x - u * a.y : v * a.x + u * a.y;
+      }
+      T* dst = which ? k_pages + (((size_t)(slot / bs) * KV + hh) * bs + slot % bs) * Dp
+                     : q_out + ((size_t)t * H + hh) * Dp;
+      dst[d] = from_f32<T>(finite_or_zero(v));
+    }
+  }
+  // values
+  for (int idx = threadIdx.x; idx < KV * Dp; idx += blockDim.x) {
+    const int g = idx / Dp, d = idx - g * Dp;
+    float v = 0.f;
+    if (d < vdim) {
+      const int c = g * vdim + d;
+      v = to_f32(row[v_off + c]) + (v_bias ? v_bias[c] : 0.f);
+      if (v_mode == 1) v_keep[(size_t)t * nv + c] = v;
+      else if (v_mode == 2) v = (1.0f - lam) * v + lam * v_keep[(size_t)t * nv + c];
+    }
+    if (slot >= 0) v_pages[((size_t)(slot / bs) * KV + g) * Dp * bs + (size_t)d * bs + slot % bs] = from_f32<T>(finite_or_zero(v));
+  }
+}
+
+extern "C" int as_whole_norm_store(const void* proj, int dtype, int ld, int q_off, int k_off, int v_off, int H, int KV,
+                                   int dim, int vdim, int Dp, const float* q_bias, const float* k_bias,
+                                   const float* v_bias, const float* qw, const float* kw, float eps, const float* cs,
+                                   int R, float* v_keep, int v_mode, float lam, const int* slots, void* q_out,
+                                   void* k_pages, void* v_pages, int bs, int store, int num_tokens,
+                                   hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (cs && (R <= 0 || (R & 1) || R > dim)) return AS_BAD_SHAPE;
+  if (H <= 0 || KV <= 0 || dim <= 0 || vdim <= 0 || Dp < dim || Dp < vdim || bs <= 0 || ld <= 0 || (!qw) != (!kw))
+    return AS_BAD_SHAPE;
+  if (v_mode < 0 || v_mode > 2 || (v_mode && !v_keep)) return AS_BAD_SHAPE;
+  if (dtype == DT_F32)
+    whole_norm_store_kernel<float><<<num_tokens, 256, 0, stream>>>(
+        (const float*)proj, ld, q_off, k_off, v_off, H, KV, dim, vdim, Dp, q_bias, k_bias, v_bias, qw, kw, eps,
+        (const float2*)cs, R, v_keep, v_mode, lam, slots, (float*)q_out, (float*)k_pages, (float*)v_pages, bs, store);
+  else if (dtype == DT_BF16)
+    whole_norm_store_kernel<bf16><<<num_tokens, 256, 0, stream>>>(
+        (const bf16*)proj, ld, q_off, k_off, v_off, H, KV, dim, vdim, Dp, q_bias, k_bias, v_bias, qw, kw, eps,
+        (const float2*)cs, R, v_keep, v_mode, lam, slots, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages, bs, store);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
 // ---- an output gate on attention heads --------------------------------------------------------
 // out[t, out_off + h * vdim + j] = scale * sigmoid(gate[t, gate_off + h * vdim + j]) * heads[t, h, j]
 // for j < vdim of the Dp coordinates a head is laid out with; gate [T, ld_gate], out [T, ld_out].
@@ -693,9 +791,9 @@ __global__ void sigmoid_gate_heads_kernel(const T* __restrict__ heads, int H, in
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
     const size_t t = idx / per;
     const int c = (int)(idx % per), h = c / vdim, j = c % vdim;
-    const float g = to_f32(gate[t * ld_gate + gate_off + c]);
     const float v = to_f32(heads[(t * H + h) * Dp + j]);
-    out[t * ld_out + out_off + c] = from_f32<T>(scale * v / (1.0f + expf(-g)));
+    const float g = gate ? 1.0f / (1.0f + expf(-to_f32(gate[t * ld_gate + gate_off + c]))) : 1.0f;  // no gate: the heads, scaled
+    out[t * ld_out + out_off + c] = from_f32<T>(scale * v * g);
   }
 }
 

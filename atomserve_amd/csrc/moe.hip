@@ -78,6 +78,9 @@ __global__ __launch_bounds__(1024) void moe_route_table_kernel(const int* __rest
 // z = router h (+ bias [experts] fp32) in fp32 (router [experts, K], h [T, K], both T-typed).  mode 0: s = sigmoid(z); a
 // token's `top` experts are those with the largest s (of equal ones the lower number first); their weights are
 // s / (sum of the chosen + 1e-20).  mode 1: the experts with the largest z, weighing the softmax over the chosen z alone.
+// mode 2: s = softmax(z) over all experts; the experts form `groups` equal groups of neighbours, a group scores its
+// largest s, and only experts of the `keep` best groups (of equal ones the lower number first) can be chosen; the `top`
+// largest s among them weigh s * scale, not renormalised.
 // pair_expert, pair_weight [T * top].  A workgroup per token: its waves take the experts four at a time, a lane 16 bytes
 // of the token's row and of the four router rows at a time (the rows stream once, coalesced), the sums meet by lane swaps
 // and the scores in LDS, where the first wave makes the choice.
@@ -101,10 +104,11 @@ template <> struct RoutePiece<bf16> {
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_scores_kernel(const T* __restrict__ h, const T* __restrict__ router,
                                                                 const float* __restrict__ bias, int mode,
+                                                                int groups, int keep, float scale,
                                                                 int K, int experts, int top, int num_tokens,
                                                                 int* __restrict__ pair_expert,
                                                                 float* __restrict__ pair_weight) {
-  extern __shared__ float scores[];  // [experts]
+  extern __shared__ float scores[];  // [experts], then [groups] group scores and [groups] marks of the kept ones
   constexpr int N = RoutePiece<T>::N;
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
   const int t = blockIdx.x;
@@ -137,13 +141,53 @@ __global__ __launch_bounds__(256) void moe_route_scores_kernel(const T* __restri
       float zs = wave_sum(z[j]);
       if (lane == 0 && e0 + j < experts) {
         if (bias) zs += bias[e0 + j];
-        scores[e0 + j] = mode == 1 ? zs : 1.0f / (1.0f + expf(-zs));
+        scores[e0 + j] = mode >= 1 ? zs : 1.0f / (1.0f + expf(-zs));
       }
     }
   }
   __syncthreads();
   if (wave) return;
   float* mine = scores;
+  if (mode == 2) {
+    float mx = -INFINITY, sum = 0.f;
+    for (int e = lane; e < experts; e += WAVE) mx = fmaxf(mx, mine[e]);
+    mx = wave_max(mx);
+    for (int e = lane; e < experts; e += WAVE) sum += expf(mine[e] - mx);
+    sum = wave_sum(sum);
+    for (int e = lane; e < experts; e += WAVE) mine[e] = expf(mine[e] - mx) / sum;
+    __builtin_amdgcn_wave_barrier();
+    if (groups > 1 && keep < groups) {
+      float* gscore = scores + experts;
+      float* gkept = gscore + groups;
+      const int per = experts / groups;
+      for (int g = lane; g < groups; g += WAVE) {
+        float m = -INFINITY;
+        for (int e = g * per; e < (g + 1) * per; ++e) m = fmaxf(m, mine[e]);
+        gscore[g] = m;
+        gkept[g] = 0.f;
+      }
+      __builtin_amdgcn_wave_barrier();
+      for (int j = 0; j < keep; ++j) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+        for (int g = lane; g < groups; g += WAVE) {
+          const float v = gscore[g];
+          if (gkept[g] == 0.f && (v > best || at == 0x7fffffff)) { best = v; at = g; }
+        }
+#pragma unroll
+        for (int off = WAVE / 2; off > 0; off >>= 1) {
+          const float ob = __shfl_xor(best, off, WAVE);
+          const int oa = __shfl_xor(at, off, WAVE);
+          if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+        }
+        if (lane == 0 && at < groups) gkept[at] = 1.f;
+        __builtin_amdgcn_wave_barrier();
+      }
+      for (int e = lane; e < experts; e += WAVE)
+        if (gkept[e / per] == 0.f) mine[e] = -INFINITY;
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
   float total = 0.f, my_score = 0.f, largest = 0.f;
   int my_expert = 0;
   for (int j = 0; j < top; ++j) {
@@ -173,7 +217,7 @@ __global__ __launch_bounds__(256) void moe_route_scores_kernel(const T* __restri
     if (lane == 0) mine[at] = -INFINITY;
     __builtin_amdgcn_wave_barrier();
   }
-  const float inv = 1.0f / (total + (mode == 1 ? 0.f : 1e-20f));
+  const float inv = mode == 2 ? scale : 1.0f / (total + (mode == 1 ? 0.f : 1e-20f));
   if (lane < top && lane < WAVE) {
     pair_expert[(size_t)t * top + lane] = my_expert;
     pair_weight[(size_t)t * top + lane] = my_score * inv;
@@ -182,18 +226,20 @@ __global__ __launch_bounds__(256) void moe_route_scores_kernel(const T* __restri
     for (int j = WAVE; j < top; ++j) pair_weight[(size_t)t * top + j] *= inv;
 }
 
-extern "C" int as_moe_route_scores(const void* h, const void* router, const float* bias, int mode, int dtype, int K,
+extern "C" int as_moe_route_scores(const void* h, const void* router, const float* bias, int mode, int groups, int keep,
+                                   float scale, int dtype, int K,
                                    int experts, int top, int num_tokens, int* pair_expert, float* pair_weight,
                                    hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
-  if (K <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts || mode < 0 || mode > 1) return AS_BAD_SHAPE;
+  if (K <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts || mode < 0 || mode > 2) return AS_BAD_SHAPE;
+  if (mode == 2 && (groups < 1 || experts % groups || keep < 1 || keep > groups || keep * (experts / groups) < top)) return AS_BAD_SHAPE;
   const int blocks = num_tokens;
-  const size_t lds = (size_t)experts * sizeof(float);
+  const size_t lds = (size_t)(experts + 2 * (groups > 0 ? groups : 0)) * sizeof(float);
   if (dtype == DT_F32)
-    moe_route_scores_kernel<float><<<blocks, 256, lds, stream>>>((const float*)h, (const float*)router, bias, mode, K, experts, top,
+    moe_route_scores_kernel<float><<<blocks, 256, lds, stream>>>((const float*)h, (const float*)router, bias, mode, groups, keep, scale, K, experts, top,
                                                                   num_tokens, pair_expert, pair_weight);
   else if (dtype == DT_BF16)
-    moe_route_scores_kernel<bf16><<<blocks, 256, lds, stream>>>((const bf16*)h, (const bf16*)router, bias, mode, K, experts, top,
+    moe_route_scores_kernel<bf16><<<blocks, 256, lds, stream>>>((const bf16*)h, (const bf16*)router, bias, mode, groups, keep, scale, K, experts, top,
                                                                  num_tokens, pair_expert, pair_weight);
   else return AS_BAD_DTYPE;
   return launch_status();

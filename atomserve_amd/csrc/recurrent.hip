@@ -198,16 +198,26 @@ template <int SL> __device__ __forceinline__ float slices_sum(float v) {
   return v;
 }
 
-template <int RPL, int SL>
+// MODE 0: the rule above.  MODE 1: a decay per head and key channel, chan [T, H, dim], on the rows of S:
+//   S <- diag(g) S, then as above; with p = S_old^T (g k), r = S_old^T (g q): u = beta (v - p), S_new = g S_old + k u^T,
+//   o = r + u (k . q).  The decays of a token go through LDS beside its key and query.
+// MODE 2: a matrix memory with exponential gates: `beta` holds the logarithm of the input gate i, `decay` that of the
+//   forget gate f, [T, H]; beside S the head keeps a normaliser n [dim] and a running maximum m (0 at the start):
+//   m' = max(f + m, i);  S' = e^(f + m - m') S + e^(i - m') k v^T;  n' = e^(f + m - m') n + e^(i - m') k;
+//   o = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6).  norm_state [slots, H, dim], max_state [slots, H].
+template <int RPL, int SL, int MODE>
 __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict__ qkv, int C, int G, int dim, int H,
                                                         int vdim, const float* __restrict__ beta,
-                                                        const float* __restrict__ decay, float* __restrict__ state,
+                                                        const float* __restrict__ decay,
+                                                        const float* __restrict__ chan, float* __restrict__ state,
+                                                        float* __restrict__ norm_state, float* __restrict__ max_state,
                                                         const int* __restrict__ row_first,
                                                         const int* __restrict__ row_len,
                                                         const int* __restrict__ row_start,
                                                         const int* __restrict__ row_slots, int writes,
                                                         float* __restrict__ out) {
-  extern __shared__ __attribute__((aligned(16))) float lds[];  // [DELTA_TB][2][dimp]: key then query of each token, dimp = SL * RPL
+  constexpr int NV = MODE == 1 ? 3 : 2;  // vectors of a token that go through LDS: key, query (, decays)
+  extern __shared__ __attribute__((aligned(16))) float lds[];  // [DELTA_TB][NV][dimp], dimp = SL * RPL
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   constexpr int CJ = WAVE / SL;
   const int col = lane / SL, slice = lane % SL;
@@ -218,13 +228,21 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
   const int first = row_first[r], len = row_len[r], slot = row_slots[r];
   const int i0 = slice * RPL;
   float S[RPL];
+  float N[MODE == 2 ? RPL : 1];
+  float m_run = 0.f;
   float* mine = state + ((size_t)(slot < 0 ? 0 : slot) * H + h) * dim * vdim;
   const bool carried = row_start[r] > 0 && slot >= 0;
 #pragma unroll
   for (int i = 0; i < RPL; ++i) S[i] = (carried && live && i0 + i < dim) ? mine[(size_t)(i0 + i) * vdim + j] : 0.f;
+  if (MODE == 2) {
+    const float* n_mine = norm_state + ((size_t)(slot < 0 ? 0 : slot) * H + h) * dim;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) N[i] = (carried && i0 + i < dim) ? n_mine[i0 + i] : 0.f;
+    m_run = carried ? max_state[(size_t)slot * H + h] : 0.f;
+  }
   const int q_col = g * dim, k_col = (G + g) * dim, v_col = 2 * G * dim + h * vdim;
-  // a round's keys and queries as 16-byte pieces: piece -> (token, key or query, four coordinates)
-  const int quads = dimp >> 2, per_token = 2 * quads, pieces = DELTA_TB * per_token;
+  // a round's keys and queries as 16-byte pieces: piece -> (token, which vector, four coordinates)
+  const int quads = dimp >> 2, per_token = NV * quads, pieces = DELTA_TB * per_token;
   const int passes = (pieces + WAVE * DELTA_STAGE - 1) / (WAVE * DELTA_STAGE);
   float4 stage[DELTA_STAGE];
   float vj[DELTA_TB], bt[DELTA_TB], gt[DELTA_TB];
@@ -234,10 +252,11 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
 #pragma unroll
     for (int u = 0; u < DELTA_STAGE; ++u) {
       const int piece = (pass * DELTA_STAGE + u) * WAVE + lane;
-      const int tt = piece / per_token, rest = piece - tt * per_token, which = rest >= quads, i = (rest - which * quads) * 4;
+      const int tt = piece / per_token, rest = piece - tt * per_token, which = rest / quads, i = (rest - which * quads) * 4;
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
       if (tt < nt && i < dim && piece < pieces) {
-        const float* src = qkv + (size_t)(first + t0 + tt) * C + (which ? q_col : k_col) + i;
+        const size_t t = (size_t)(first + t0 + tt);
+        const float* src = which == 2 ? chan + (t * H + h) * dim + i : qkv + t * C + (which ? q_col : k_col) + i;
         if (whole) {
           v = *reinterpret_cast<const float4*>(src);
         } else {  // widths that are no multiples of 4: value by value
@@ -257,7 +276,7 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
       const size_t t = (size_t)first + t0 + (tt < nt ? tt : 0);
       vj[tt] = live ? qkv[t * C + v_col + j] : 0.f;
       bt[tt] = beta[t * H + h];
-      gt[tt] = decay[t * H + h];
+      gt[tt] = MODE == 1 ? 1.f : decay[t * H + h];
     }
   };
   auto put = [&](int pass) {
@@ -291,14 +310,46 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
     for (int tt = 0; tt < DELTA_TB; ++tt) {
       if (tt < nt) {
         // this lane's slice of the token's key and query, 16 bytes at a time (i0 is a multiple of 8)
-        const float4* k4 = reinterpret_cast<const float4*>(lds + tt * 2 * dimp + i0);
-        const float4* q4 = reinterpret_cast<const float4*>(lds + tt * 2 * dimp + dimp + i0);
+        const float4* k4 = reinterpret_cast<const float4*>(lds + tt * NV * dimp + i0);
+        const float4* q4 = reinterpret_cast<const float4*>(lds + tt * NV * dimp + dimp + i0);
         float kk[RPL], qq[RPL];
 #pragma unroll
         for (int i = 0; i < RPL / 4; ++i) {
           const float4 a = k4[i], b = q4[i];
           kk[4 * i] = a.x; kk[4 * i + 1] = a.y; kk[4 * i + 2] = a.z; kk[4 * i + 3] = a.w;
           qq[4 * i] = b.x; qq[4 * i + 1] = b.y; qq[4 * i + 2] = b.z; qq[4 * i + 3] = b.w;
+        }
+        if (MODE == 2) {
+          const float fl = g_now[tt], il = b_now[tt];
+          const float m_new = fmaxf(fl + m_run, il);
+          const float keep = expf(fl + m_run - m_new), take = expf(il - m_new);
+          m_run = m_new;
+          const float tv = take * v_now[tt];
+          float num = 0.f, nq = 0.f, num2 = 0.f, nq2 = 0.f;
+#pragma unroll
+          for (int i = 0; i < RPL; i += 2) {
+            S[i] = fmaf(kk[i], tv, keep * S[i]);
+            N[i] = fmaf(kk[i], take, keep * N[i]);
+            num = fmaf(S[i], qq[i], num);
+            nq = fmaf(N[i], qq[i], nq);
+            S[i + 1] = fmaf(kk[i + 1], tv, keep * S[i + 1]);
+            N[i + 1] = fmaf(kk[i + 1], take, keep * N[i + 1]);
+            num2 = fmaf(S[i + 1], qq[i + 1], num2);
+            nq2 = fmaf(N[i + 1], qq[i + 1], nq2);
+          }
+          num = slices_sum<SL>(num + num2);
+          nq = slices_sum<SL>(nq + nq2);
+          if (live && slice == 0)
+            out[((size_t)(first + t0 + tt) * H + h) * vdim + j] = num / (fmaxf(fabsf(nq), expf(-m_new)) + 1e-6f);
+          continue;
+        }
+        if (MODE == 1) {  // the decays act on the rows of the old state
+          const float4* g4 = reinterpret_cast<const float4*>(lds + tt * NV * dimp + 2 * dimp + i0);
+#pragma unroll
+          for (int i = 0; i < RPL / 4; ++i) {
+            const float4 a = g4[i];
+            S[4 * i] *= a.x; S[4 * i + 1] *= a.y; S[4 * i + 2] *= a.z; S[4 * i + 3] *= a.w;
+          }
         }
         float p = 0.f, rr = 0.f, kq = 0.f, p2 = 0.f, rr2 = 0.f, kq2 = 0.f;  // two chains each: half the dependent steps
 #pragma unroll
@@ -326,18 +377,28 @@ __global__ __launch_bounds__(64) void delta_scan_kernel(const float* __restrict_
     for (int i = 0; i < RPL; ++i)
       if (i0 + i < dim) mine[(size_t)(i0 + i) * vdim + j] = S[i];
   }
+  if (MODE == 2 && writes && slot >= 0 && blockIdx.z == 0 && col == 0) {  // every column group keeps the same n and m: one writes
+    float* n_mine = norm_state + ((size_t)slot * H + h) * dim;
+#pragma unroll
+    for (int i = 0; i < RPL; ++i)
+      if (i0 + i < dim) n_mine[i0 + i] = N[i];
+    if (slice == 0) max_state[(size_t)slot * H + h] = m_run;
+  }
 }
 
-extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int vdim, const float* beta,
-                             const float* decay, float* state, const int* row_first, const int* row_len,
-                             const int* row_start, const int* row_slots, int writes, float* out, int num_rows,
-                             int force_slices, hipStream_t stream) {
+template <int MODE>
+static int launch_delta_scan(const float* qkv, int C, int G, int dim, int H, int vdim, const float* beta,
+                             const float* decay, const float* chan, float* state, float* norm_state, float* max_state,
+                             const int* row_first, const int* row_len, const int* row_start, const int* row_slots,
+                             int writes, float* out, int num_rows, int force_slices, hipStream_t stream) {
   if (num_rows <= 0) return AS_OK;
   if (G <= 0 || H <= 0 || H % G || dim <= 0 || vdim <= 0 || C < 2 * G * dim + H * vdim || H > 65535)
     return AS_BAD_SHAPE;
   if (dim > 16 * 64) return AS_BAD_SHAPE;  // sixteen slices of 64 rows
   int slices = 1;
   while ((dim + slices - 1) / slices > 64) slices *= 2;  // a lane keeps at most 64 rows of its column
+  if (MODE == 2)  // the normaliser's rows lie beside the state's: half as many to a lane
+    while ((dim + slices - 1) / slices > 32) slices *= 2;
   // few rows and heads: narrower column groups (more slices of fewer rows) until the waves fill the GPU
   while (slices < 16 && (dim + 2 * slices - 1) / (2 * slices) >= 8 &&
          (long)num_rows * H * ((vdim + WAVE / slices - 1) / (WAVE / slices)) < 8L * compute_units())
@@ -347,14 +408,17 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
       return AS_BAD_SHAPE;
     slices = force_slices;
   }
+  if (slices > 16) return AS_BAD_SHAPE;
   const int rows_per_lane = (dim + slices - 1) / slices;
   const int RPL = rows_per_lane <= 8 ? 8 : rows_per_lane <= 16 ? 16 : rows_per_lane <= 32 ? 32 : 64;
   const int CJ = WAVE / slices;
   dim3 grid(num_rows, H, (vdim + CJ - 1) / CJ);
-  const size_t lds = (size_t)DELTA_TB * 2 * slices * RPL * sizeof(float);
-#define LAUNCH(R, SLV)                                                                                          \
-  delta_scan_kernel<R, SLV><<<grid, 64, lds, stream>>>(qkv, C, G, dim, H, vdim, beta, decay, state, row_first,  \
-                                                       row_len, row_start, row_slots, writes, out)
+  const size_t lds = (size_t)DELTA_TB * (MODE == 1 ? 3 : 2) * slices * RPL * sizeof(float);
+  if (lds > 64 * 1024) return AS_BAD_SHAPE;
+#define LAUNCH(R, SLV)                                                                                            \
+  delta_scan_kernel<R, SLV, MODE><<<grid, 64, lds, stream>>>(qkv, C, G, dim, H, vdim, beta, decay, chan, state,   \
+                                                             norm_state, max_state, row_first, row_len, row_start, \
+                                                             row_slots, writes, out)
 #define LAUNCH_SL(R)              \
   do {                            \
     if (slices == 1) LAUNCH(R, 1);      \
@@ -372,38 +436,177 @@ extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int
   return launch_status();
 }
 
+extern "C" int as_delta_scan(const float* qkv, int C, int G, int dim, int H, int vdim, const float* beta,
+                             const float* decay, float* state, const int* row_first, const int* row_len,
+                             const int* row_start, const int* row_slots, int writes, float* out, int num_rows,
+                             int force_slices, hipStream_t stream) {
+  return launch_delta_scan<0>(qkv, C, G, dim, H, vdim, beta, decay, nullptr, state, nullptr, nullptr, row_first, row_len,
+                              row_start, row_slots, writes, out, num_rows, force_slices, stream);
+}
+
+// The same rule with a decay per head and key channel: chan [T, H, dim].
+extern "C" int as_delta_scan_channels(const float* qkv, int C, int G, int dim, int H, int vdim, const float* beta,
+                                      const float* chan, float* state, const int* row_first, const int* row_len,
+                                      const int* row_start, const int* row_slots, int writes, float* out,
+                                      int num_rows, int force_slices, hipStream_t stream) {
+  if (!chan) return AS_BAD_SHAPE;
+  return launch_delta_scan<1>(qkv, C, G, dim, H, vdim, beta, nullptr, chan, state, nullptr, nullptr, row_first, row_len,
+                              row_start, row_slots, writes, out, num_rows, force_slices, stream);
+}
+
+// The matrix memory: qkv [T, C] holds H query heads (already times dim^(-1/2)), H key heads and H value heads.
+extern "C" int as_memory_scan(const float* qkv, int C, int dim, int H, int vdim, const float* i_log, const float* f_log,
+                              float* state, float* norm_state, float* max_state, const int* row_first,
+                              const int* row_len, const int* row_start, const int* row_slots, int writes, float* out,
+                              int num_rows, int force_slices, hipStream_t stream) {
+  if (!norm_state || !max_state) return AS_BAD_SHAPE;
+  return launch_delta_scan<2>(qkv, C, H, dim, H, vdim, i_log, f_log, nullptr, state, norm_state, max_state, row_first,
+                              row_len, row_start, row_slots, writes, out, num_rows, force_slices, stream);
+}
+
 // After the scan: every head's output over its root mean square (over vdim, eps inside the root), times
-// a weight [vdim] shared by the heads, times silu of the gate projection's output (proj [T, ld] at
-// g_off, laid out heads x vdim): the input of the output projection, [T, H * vdim] in T.
+// a weight (w [vdim] shared by the heads with w_stride 0, w [H, vdim] with w_stride vdim), times silu (gate_act 0)
+// or sigmoid (1) of a gate projection's output (gate [T, ld] at g_off, laid out heads x vdim), times scale: the
+// input of the output projection, act [T, ld_out] from column out_off on.
 template <typename T, typename W>
 __global__ __launch_bounds__(64) void delta_finish_kernel(const float* __restrict__ o, int H, int vdim,
-                                                          const W* __restrict__ w, float eps,
-                                                          const T* __restrict__ proj, int ld, int g_off,
-                                                          T* __restrict__ act) {
+                                                          const W* __restrict__ w, int w_stride, float eps,
+                                                          const T* __restrict__ gate, int ld, int g_off, int gate_act,
+                                                          float scale, T* __restrict__ act, int ld_out, int out_off) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* x = o + ((size_t)t * H + h) * vdim;
   float ss = 0.f;
   for (int d = lane; d < vdim; d += WAVE) ss += x[d] * x[d];
   ss = wave_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+  const float inv = scale / sqrtf(ss / (float)vdim + eps);
   for (int d = lane; d < vdim; d += WAVE) {
-    const float gate = to_f32(proj[(size_t)t * ld + g_off + h * vdim + d]);
-    act[((size_t)t * H + h) * vdim + d] = from_f32<T>(x[d] * inv * to_f32(w[d]) * siluf_(gate));
+    const float z = to_f32(gate[(size_t)t * ld + g_off + h * vdim + d]);
+    const float gv = gate_act == 1 ? sigmoidf_(z) : siluf_(z);
+    act[(size_t)t * ld_out + out_off + h * vdim + d] = from_f32<T>(x[d] * inv * to_f32(w[(size_t)h * w_stride + d]) * gv);
   }
 }
 
-extern "C" int as_delta_finish(const float* o, int H, int vdim, const void* w, int w_dtype, float eps, const void* proj,
-                               int dtype, int ld, int g_off, void* act, int num_tokens, hipStream_t stream) {
+extern "C" int as_delta_finish(const float* o, int H, int vdim, const void* w, int w_dtype, int w_per_head, float eps,
+                               const void* gate, int dtype, int ld, int g_off, int gate_act, float scale, void* act,
+                               int ld_out, int out_off, int num_tokens, hipStream_t stream) {
   if (num_tokens <= 0) return AS_OK;
-  if (H <= 0 || H > 65535 || vdim <= 0) return AS_BAD_SHAPE;
+  if (H <= 0 || H > 65535 || vdim <= 0 || gate_act < 0 || gate_act > 1 || ld < g_off + H * vdim ||
+      ld_out < out_off + H * vdim)
+    return AS_BAD_SHAPE;
   dim3 grid(num_tokens, H);
-#define LAUNCH(T, W)                                                                                             \
-  delta_finish_kernel<T, W><<<grid, 64, 0, stream>>>(o, H, vdim, (const W*)w, eps, (const T*)proj, ld, g_off, (T*)act)
+  const int w_stride = w_per_head ? vdim : 0;
+#define LAUNCH(T, W)                                                                                               \
+  delta_finish_kernel<T, W><<<grid, 64, 0, stream>>>(o, H, vdim, (const W*)w, w_stride, eps, (const T*)gate, ld,  \
+                                                     g_off, gate_act, scale, (T*)act, ld_out, out_off)
   if (dtype == DT_F32 && w_dtype == DT_F32) LAUNCH(float, float);
   else if (dtype == DT_BF16 && w_dtype == DT_BF16) LAUNCH(bf16, bf16);
   else if (dtype == DT_BF16 && w_dtype == DT_F32) LAUNCH(bf16, float);
   else return AS_BAD_DTYPE;
 #undef LAUNCH
+  return launch_status();
+}
+
+// Before the scan with a decay per channel: unit vectors as in delta_prepare; beta = sigmoid(proj[t, b_off + h]);
+// chan[t, h, d] = exp(-exp(a_log[h]) * softplus(steps[t, a_off + h * dim + d] + dt_bias[h * dim + d])), `steps` being
+// the output of the step sizes' second projection, [T, ld_s].  a_log and dt_bias fp32.
+template <typename T>
+__global__ __launch_bounds__(256) void delta_prepare_channels_kernel(float* __restrict__ qkv, int C, int G, int dim, int H,
+                                                                     const T* __restrict__ proj, int ld, int b_off,
+                                                                     const T* __restrict__ steps, int ld_s, int a_off,
+                                                                     const float* __restrict__ a_log,
+                                                                     const float* __restrict__ dt_bias,
+                                                                     float* __restrict__ beta, float* __restrict__ chan) {
+  const int t = blockIdx.x, lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
+  float* row = qkv + (size_t)t * C;
+  for (int head = blockIdx.y * waves + wave; head < 2 * G; head += gridDim.y * waves) {
+    float* x = row + (size_t)head * dim;  // query heads first, then key heads
+    float ss = 0.f;
+    for (int d = lane; d < dim; d += WAVE) ss += x[d] * x[d];
+    ss = wave_sum(ss);
+    float f = 1.0f / sqrtf(ss + 1e-6f);
+    if (head < G) f *= 1.0f / sqrtf((float)dim);
+    for (int d = lane; d < dim; d += WAVE) x[d] *= f;
+  }
+  for (int h = blockIdx.y * blockDim.x + threadIdx.x; h < H; h += gridDim.y * blockDim.x)
+    beta[(size_t)t * H + h] = sigmoidf_(to_f32(proj[(size_t)t * ld + b_off + h]));
+  const int HD = H * dim;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < HD; c += gridDim.y * blockDim.x) {
+    const float a = to_f32(steps[(size_t)t * ld_s + a_off + c]);
+    chan[(size_t)t * HD + c] = expf(-expf(a_log[c / dim]) * softplusf_(a + dt_bias[c]));
+  }
+}
+
+extern "C" int as_delta_prepare_channels(float* qkv, int C, int G, int dim, int H, const void* proj, int dtype, int ld,
+                                         int b_off, const void* steps, int ld_s, int a_off, const float* a_log,
+                                         const float* dt_bias, float* beta, float* chan, int num_tokens,
+                                         hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (G <= 0 || dim <= 0 || H <= 0 || C < 2 * G * dim || ld < b_off + H || ld_s < a_off + H * dim) return AS_BAD_SHAPE;
+  int across = num_tokens >= 512 ? 1 : (H * dim + 255) / 256;
+  if (across > 64) across = 64;
+  dim3 grid(num_tokens, across);
+  if (dtype == DT_F32)
+    delta_prepare_channels_kernel<float><<<grid, 256, 0, stream>>>(qkv, C, G, dim, H, (const float*)proj, ld, b_off,
+                                                                   (const float*)steps, ld_s, a_off, a_log, dt_bias,
+                                                                   beta, chan);
+  else if (dtype == DT_BF16)
+    delta_prepare_channels_kernel<bf16><<<grid, 256, 0, stream>>>(qkv, C, G, dim, H, (const bf16*)proj, ld, b_off,
+                                                                  (const bf16*)steps, ld_s, a_off, a_log, dt_bias, beta,
+                                                                  chan);
+  else return AS_BAD_DTYPE;
+  return launch_status();
+}
+
+// Before the scan of a matrix memory: proj [T, ld] holds H query heads at q_off, H key heads at k_off (`dim` wide) and
+// H value heads at v_off (`vdim` wide), and the gates' logits at i_off and f_off [H].  qkv fp32 [T, 2 H dim + H vdim]
+// receives the queries times dim^(-1/2), the keys and the values; i_log = cap tanh((z_i + b_i) / cap), f_log =
+// logsigmoid(cap tanh((z_f + b_f) / cap)), both [T, H]; biases fp32 [H].
+__device__ __forceinline__ float log_sigmoidf_(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void memory_prepare_kernel(const T* __restrict__ proj, int ld, int q_off, int k_off,
+                                                             int v_off, int i_off, int f_off, int H, int dim, int vdim,
+                                                             const float* __restrict__ i_bias,
+                                                             const float* __restrict__ f_bias, float cap,
+                                                             float* __restrict__ qkv, float* __restrict__ i_log,
+                                                             float* __restrict__ f_log) {
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * ld;
+  const int HD = H * dim, C = 2 * HD + H * vdim;
+  const float qs = 1.0f / sqrtf((float)dim);
+  float* dst = qkv + (size_t)t * C;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
+    float v;
+    if (c < HD) v = to_f32(row[q_off + c]) * qs;
+    else if (c < 2 * HD) v = to_f32(row[k_off + c - HD]);
+    else v = to_f32(row[v_off + c - 2 * HD]);
+    dst[c] = v;
+  }
+  for (int h = blockIdx.y * blockDim.x + threadIdx.x; h < H; h += gridDim.y * blockDim.x) {
+    const float zi = to_f32(row[i_off + h]) + i_bias[h], zf = to_f32(row[f_off + h]) + f_bias[h];
+    i_log[(size_t)t * H + h] = cap * tanhf(zi / cap);
+    f_log[(size_t)t * H + h] = log_sigmoidf_(cap * tanhf(zf / cap));
+  }
+}
+
+extern "C" int as_memory_prepare(const void* proj, int dtype, int ld, int q_off, int k_off, int v_off, int i_off,
+                                 int f_off, int H, int dim, int vdim, const float* i_bias, const float* f_bias,
+                                 float cap, float* qkv, float* i_log, float* f_log, int num_tokens,
+                                 hipStream_t stream) {
+  if (num_tokens <= 0) return AS_OK;
+  if (H <= 0 || dim <= 0 || vdim <= 0 || !(cap > 0.f) || ld < q_off + H * dim || ld < k_off + H * dim ||
+      ld < v_off + H * vdim || ld < i_off + H || ld < f_off + H)
+    return AS_BAD_SHAPE;
+  int across = num_tokens >= 512 ? 1 : ((2 * dim + vdim) * H + 255) / 256;
+  if (across > 64) across = 64;
+  dim3 grid(num_tokens, across);
+  if (dtype == DT_F32)
+    memory_prepare_kernel<float><<<grid, 256, 0, stream>>>((const float*)proj, ld, q_off, k_off, v_off, i_off, f_off, H,
+                                                           dim, vdim, i_bias, f_bias, cap, qkv, i_log, f_log);
+  else if (dtype == DT_BF16)
+    memory_prepare_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)proj, ld, q_off, k_off, v_off, i_off, f_off, H,
+                                                          dim, vdim, i_bias, f_bias, cap, qkv, i_log, f_log);
+  else return AS_BAD_DTYPE;
   return launch_status();
 }
 

@@ -22,7 +22,7 @@ FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]  # fmt: skip
 HEADERS = ["common.h", "no_alloc.h"]
 LIBRARIES = ("elementwise", "attention", "attention_mix", "gemm", "sampling", "blas", "recurrent", "moe", "layer_ops",
-             "linear_attention", "latent")
+             "linear_attention", "latent", "streams")
 LINK = {"blas": ["-lhipblaslt"]}  # what a library links beside the HIP runtime
 
 

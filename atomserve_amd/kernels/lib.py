@@ -29,17 +29,23 @@ SIGNATURES = {
     "as_head_norm_store": ("elementwise", [P, I, I, I, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, I, I, P, I, P]),
     "as_gated_add_norm": ("elementwise", [P, P, P, I, I, I, P, F, P, P, I, F, P, I, I, I, I, P, P, P]),
     "as_relu2": ("elementwise", [P, I, I, I, P, I, I, P]),
+    "as_whole_norm_store": ("elementwise", [P, I, I, I, I, I, I, I, I, I, I, P, P, P, P, P, F, P, I, P, I, F, P, P, P, P, I, I, I, P]),
+    "as_streams_step": ("streams", [P, P, I, I, P, I, P, P, F, P, P, F, P, P, I, P]),
     "as_sigmoid_gate_heads": ("elementwise", [P, I, I, I, I, P, I, I, F, P, I, I, I, P]),
     "as_short_conv": ("recurrent", [P, I, I, I, I, P, P, P, I, I, I, P, P, P, P, P, P, P, I, I, I, P]),
     "as_delta_prepare": ("recurrent", [P, I, I, I, I, P, I, I, I, I, P, P, I, P, P, I, P]),
     "as_delta_scan": ("recurrent", [P, I, I, I, I, I, P, P, P, P, P, P, P, I, P, I, I, P]),
-    "as_delta_finish": ("recurrent", [P, I, I, P, I, F, P, I, I, I, P, I, P]),
+    "as_delta_finish": ("recurrent", [P, I, I, P, I, I, F, P, I, I, I, I, F, P, I, I, I, P]),
+    "as_delta_scan_channels": ("recurrent", [P, I, I, I, I, I, P, P, P, P, P, P, P, I, P, I, I, P]),
+    "as_delta_prepare_channels": ("recurrent", [P, I, I, I, I, P, I, I, I, P, I, I, P, P, P, P, I, P]),
+    "as_memory_prepare": ("recurrent", [P, I, I, I, I, I, I, I, I, I, I, P, P, F, P, P, P, I, P]),
+    "as_memory_scan": ("recurrent", [P, I, I, I, I, P, P, P, P, P, P, P, P, P, I, P, I, I, P]),
     "as_rglru_gates": ("recurrent", [P, I, I, P, P, P, P, P, I, F, P, P, I, P]),
     "as_rglru_scan": ("recurrent", [P, P, I, P, I, I, I, P, I, F, P, P, P, P, P, I, P, I, I, I, P]),
     "as_moe_route_table": ("moe", [P, P, I, I, I, I, P, P, P, I, P]),
     "as_moe_gemm": ("moe", [P, I, I, P, I, I, I, P, P, P, I, P, I, F, P]),
     "as_moe_combine": ("moe", [P, I, F, I, P, I, I, P, P, P]),
-    "as_moe_route_scores": ("moe", [P, P, P, I, I, I, I, I, I, P, P, P]),
+    "as_moe_route_scores": ("moe", [P, P, P, I, I, I, F, I, I, I, I, I, P, P, P]),
     "as_group_norm": ("layer_ops", [P, P, P, P, F, I, P, I, I, I, I, P]),
     "as_group_norm_shift": ("layer_ops", [P, P, P, F, I, P, P, P, P, P, P, P, I, I, I, I, P]),
     "as_depth_average": ("layer_ops", [P, P, I, P, P, I, c_longlong, P]),

@@ -1082,6 +1082,90 @@ def head_norm_store(proj, q_off, k_off, v_off, num_heads, num_kv_heads, dim, vdi
          _ptr(cos_sin), R, _stream())  # fmt: skip
 
 
+def whole_norm_store(proj, q_off, k_off, v_off, num_heads, num_kv_heads, dim, vdim, slots, q_out, k_pages, v_pages,
+                     store_kv=True, biases=None, gains=None, eps: float = 0.0, cos_sin=None, v_keep=None,
+                     v_mode: str = "none", lam: float = 0.0) -> None:  # fmt: skip
+    """`head_norm_store` for heads that are normed over their whole projection.  biases: (q [H dim], k [KV dim], v [KV
+    vdim]) fp32, added to the projection's output first, or None.  gains: (q [H dim], k [KV dim]) fp32: queries and keys
+    are divided by the root mean square over ALL their heads (eps inside the root) and multiplied by the gains; None: no
+    norm.  cos_sin: the rotation (after the norm), as in `head_norm_store`.  v_mode "keep": the values (bias added) are
+    also written to v_keep fp32 [T, KV vdim]; "mix": (1 - lam) v + lam v_keep[t] is stored instead of v."""
+    _check(proj, "proj", (F32, BF16), (None, None))
+    T, ld = proj.shape
+    H, KV = num_heads, num_kv_heads
+    _check(q_out, "q_out", proj.dtype, (T, H, None))
+    Dp = q_out.shape[2]
+    if Dp < max(dim, vdim) or min(q_off, k_off, v_off) < 0 or q_off + H * dim > ld or k_off + KV * dim > ld \
+            or v_off + KV * vdim > ld:  # fmt: skip
+        raise KernelError("whole_norm_store: heads lie outside the projection's columns or the padded head width")
+    qb = kb = vb = qw = kw = None
+    if biases is not None:
+        qb, kb, vb = biases
+        for name, t, n in (("q bias", qb, H * dim), ("k bias", kb, KV * dim), ("v bias", vb, KV * vdim)):
+            _check(t, name, F32, (n,))
+    if gains is not None:
+        qw, kw = gains
+        _check(qw, "q gain", F32, (H * dim,))
+        _check(kw, "k gain", F32, (KV * dim,))
+    bs = 1
+    if store_kv:
+        _check(slots, "slots", I32, (T,))
+        _check(k_pages, "k_pages", proj.dtype, (None, KV, None, Dp))
+        bs = k_pages.shape[2]
+        _check(v_pages, "v_pages", proj.dtype, (k_pages.shape[0], KV, Dp, bs))
+    R = 0
+    if cos_sin is not None:
+        _check(cos_sin, "cos_sin", F32, (T, None, 2))
+        R = 2 * cos_sin.shape[1]
+        if R > dim or R < 2:
+            raise KernelError(f"whole_norm_store: {R} turned coordinates in a head of {dim}")
+    modes = {"none": 0, "keep": 1, "mix": 2}
+    if v_mode not in modes:
+        raise KernelError(f"whole_norm_store: values are handled as one of {sorted(modes)}, not {v_mode!r}")
+    if modes[v_mode]:
+        _check(v_keep, "v_keep", F32, (T, KV * vdim))
+    call("as_whole_norm_store", _ptr(proj), _DT[proj.dtype], ld, q_off, k_off, v_off, H, KV, dim, vdim, Dp, _ptr(qb),
+         _ptr(kb), _ptr(vb), _ptr(qw), _ptr(kw), float(eps), _ptr(cos_sin), R, _ptr(v_keep) if modes[v_mode] else 0,
+         modes[v_mode], float(lam), _ptr(slots) if store_kv else 0, _ptr(q_out), _ptr(k_pages) if store_kv else 0,
+         _ptr(v_pages) if store_kv else 0, bs, int(bool(store_kv)), T, _stream())  # fmt: skip
+
+
+STREAMS_MAX = 8
+
+
+def streams_step(xs, first=None, y=None, mix=None, out_c=None, mult: float = 1.0, in_c=None, gain=None, eps: float = 0.0,
+                 normed=None, total=None) -> None:  # fmt: skip
+    """One step between two parts of a model with several residual streams xs fp32 [T, S, n] (updated in place).
+    first [T, n] fp32: the streams do not exist yet, all of them are `first`.  y [T, n] (compute dtype): the pending
+    write xs[:, r] <- sum_s mix[s, r] xs[:, s] + mult out_c[r] y (mix fp32 [S, S], None: the identity; out_c fp32 [S]).
+    in_c fp32 [S] with gain fp32 [n] and normed [T, n] (compute dtype): normed = rmsnorm(sum_s in_c[s] xs[:, s]) * gain.
+    total fp32 [T, n]: receives sum_s xs[:, s]."""
+    _check(xs, "xs", F32, (None, None, None))
+    T, S, n = xs.shape
+    if not 1 <= S <= STREAMS_MAX:
+        raise KernelError(f"1 to {STREAMS_MAX} streams, not {S}")
+    dtype = None
+    if first is not None:
+        _check(first, "first", F32, (T, n))
+    if y is not None:
+        _check(y, "y", (F32, BF16), (T, n))
+        dtype = y.dtype
+        _check(out_c, "out_c", F32, (S,))
+        if mix is not None:
+            _check(mix, "mix", F32, (S, S))
+    if (in_c is None) != (normed is None):
+        raise KernelError("streams_step: the read's weights and the normed rows come together")
+    if normed is not None:
+        _check(normed, "normed", (F32, BF16) if dtype is None else dtype, (T, n))
+        dtype = normed.dtype
+        _check(in_c, "in_c", F32, (S,))
+        _check(gain, "gain", F32, (n,))
+    if total is not None:
+        _check(total, "total", F32, (T, n))
+    call("as_streams_step", _ptr(xs), _ptr(first), S, n, _ptr(y), _DT[dtype if dtype is not None else F32], _ptr(mix),
+         _ptr(out_c), float(mult), _ptr(in_c), _ptr(gain), float(eps), _ptr(normed), _ptr(total), T, _stream())  # fmt: skip
+
+
 def gated_add_norm(x, y, gate, gate_off, bias, mult, weight, eps, out, rows=None, update_x=True, other=None,
                    join=None) -> None:  # fmt: skip
     """The fp32 stream x [T, n] takes a part's gated, scaled output and is normed, in one kernel:
@@ -1269,14 +1353,20 @@ def attn_headmix(q, k_pages, v_pages, items, tile: int, positions, tok_row, bloc
 
 
 def sigmoid_gate_heads(heads, vdim, gate, gate_off, scale, out, out_off) -> None:
-    """out[t, out_off + h * vdim + j] = scale * sigmoid(gate[t, gate_off + h * vdim + j]) * heads[t, h, j], j < vdim."""
+    """out[t, out_off + h * vdim + j] = scale * sigmoid(gate[t, gate_off + h * vdim + j]) * heads[t, h, j], j < vdim;
+    gate None: scale * heads, laid side by side."""
     _check(heads, "heads", (F32, BF16), (None, None, None))
     T, H, Dp = heads.shape
-    _check(gate, "gate", heads.dtype, (T, None))
     _check(out, "out", heads.dtype, (T, None))
-    if vdim > Dp or gate_off < 0 or gate_off + H * vdim > gate.shape[1] or out_off < 0 or out_off + H * vdim > out.shape[1]:
-        raise KernelError("sigmoid_gate_heads: columns outside the gate or the output")
-    call("as_sigmoid_gate_heads", _ptr(heads), _DT[heads.dtype], H, vdim, Dp, _ptr(gate), gate.shape[1], gate_off,
+    ld_gate = 0
+    if gate is not None:
+        _check(gate, "gate", heads.dtype, (T, None))
+        ld_gate = gate.shape[1]
+        if gate_off < 0 or gate_off + H * vdim > ld_gate:
+            raise KernelError("sigmoid_gate_heads: columns outside the gate")
+    if vdim > Dp or out_off < 0 or out_off + H * vdim > out.shape[1]:
+        raise KernelError("sigmoid_gate_heads: columns outside the output")
+    call("as_sigmoid_gate_heads", _ptr(heads), _DT[heads.dtype], H, vdim, Dp, _ptr(gate), ld_gate, gate_off,
          float(scale), _ptr(out), out.shape[1], out_off, T, _stream())  # fmt: skip
 
 
@@ -1374,18 +1464,107 @@ def delta_scan(qkv, num_kv_heads, dim, num_heads, vdim, beta, decay, state, step
          _ptr(row_len), _ptr(row_start), _ptr(row_slots), int(bool(writes)), _ptr(out), R, int(slices), _stream())  # fmt: skip
 
 
-def delta_finish(o, weight, eps, proj, g_off, act) -> None:
-    """act[t, h * vdim + j] = o[t, h, j] / rms(o[t, h]) * weight[j] * silu(proj[t, g_off + h * vdim + j])."""
+def delta_finish(o, weight, eps, proj, g_off, act, gate="silu", scale: float = 1.0, out_off: int = 0) -> None:
+    """act[t, out_off + h * vdim + j] = scale * o[t, h, j] / rms(o[t, h]) * weight * gate(proj[t, g_off + h * vdim + j]);
+    weight [vdim] (shared by the heads) or [H, vdim]; gate "silu" or "sigmoid"; act [T, >= out_off + H * vdim]."""
     _check(o, "o", F32, (None, None, None))
     T, H, vdim = o.shape
     _check(proj, "proj", (F32, BF16), (T, None))
     if g_off < 0 or g_off + H * vdim > proj.shape[1]:
         raise KernelError("delta_finish: the gate lies outside the projection's columns")
+    if gate not in ("silu", "sigmoid"):
+        raise KernelError(f"delta_finish: a gate is 'silu' or 'sigmoid', not {gate!r}")
     w_dtype = _vector_dtype(proj.dtype, weight)
-    _check(weight, "weight", w_dtype, (vdim,))
-    _check(act, "act", proj.dtype, (T, H * vdim))
-    call("as_delta_finish", _ptr(o), H, vdim, _ptr(weight), _DT[w_dtype], float(eps), _ptr(proj), _DT[proj.dtype],
-         proj.shape[1], g_off, _ptr(act), T, _stream())  # fmt: skip
+    per_head = weight.dim() == 2
+    _check(weight, "weight", w_dtype, (H, vdim) if per_head else (vdim,))
+    _check(act, "act", proj.dtype, (T, None))
+    if out_off < 0 or out_off + H * vdim > act.shape[1]:
+        raise KernelError("delta_finish: the heads lie outside the output's columns")
+    call("as_delta_finish", _ptr(o), H, vdim, _ptr(weight), _DT[w_dtype], int(per_head), float(eps), _ptr(proj),
+         _DT[proj.dtype], proj.shape[1], g_off, int(gate == "sigmoid"), float(scale), _ptr(act), act.shape[1], out_off,
+         T, _stream())  # fmt: skip
+
+
+def delta_prepare_channels(qkv, num_kv_heads, dim, num_heads, proj, b_off, steps, a_off, a_log, dt_bias, beta, chan) -> None:
+    """As `delta_prepare` for a rule with a decay per head and key channel: chan [T, H, dim] =
+    exp(-exp(a_log[h]) * softplus(steps[:, a_off + h * dim + d] + dt_bias[h * dim + d])); a_log [H], dt_bias [H * dim] fp32."""
+    _check(qkv, "qkv", F32, (None, None))
+    T, C = qkv.shape
+    G, H = num_kv_heads, num_heads
+    _check(proj, "proj", (F32, BF16), (T, None))
+    _check(steps, "steps", proj.dtype, (T, None))
+    if C < 2 * G * dim or b_off < 0 or b_off + H > proj.shape[1] or a_off < 0 or a_off + H * dim > steps.shape[1]:
+        raise KernelError("delta_prepare_channels: heads outside the convolution's channels or the projections' columns")
+    _check(a_log, "a_log", F32, (H,))
+    _check(dt_bias, "dt_bias", F32, (H * dim,))
+    _check(beta, "beta", F32, (T, H))
+    _check(chan, "chan", F32, (T, H, dim))
+    call("as_delta_prepare_channels", _ptr(qkv), C, G, dim, H, _ptr(proj), _DT[proj.dtype], proj.shape[1], b_off,
+         _ptr(steps), steps.shape[1], a_off, _ptr(a_log), _ptr(dt_bias), _ptr(beta), _ptr(chan), T, _stream())  # fmt: skip
+
+
+def delta_scan_channels(qkv, num_kv_heads, dim, num_heads, vdim, beta, chan, state, step_rows, out, writes=True, slices=0) -> None:
+    """`delta_scan` with a decay per head and key channel, chan fp32 [T, H, dim], acting on the rows of S:
+    S <- diag(chan) S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q."""
+    _check(qkv, "qkv", F32, (None, None))
+    T, C = qkv.shape
+    G, H = num_kv_heads, num_heads
+    if H % G or C != 2 * G * dim + H * vdim:
+        raise KernelError(f"delta_scan_channels: {C} channels are not 2 x {G} x {dim} + {H} x {vdim}")
+    _check(beta, "beta", F32, (T, H))
+    _check(chan, "chan", F32, (T, H, dim))
+    _check(state, "state", F32, (None, H, dim, vdim))
+    _check(out, "out", F32, (T, H, vdim))
+    R = _check_rows((None, *step_rows[1:]), 0)
+    _, row_first, row_len, row_start, row_slots = step_rows
+    call("as_delta_scan_channels", _ptr(qkv), C, G, dim, H, vdim, _ptr(beta), _ptr(chan), _ptr(state), _ptr(row_first),
+         _ptr(row_len), _ptr(row_start), _ptr(row_slots), int(bool(writes)), _ptr(out), R, int(slices), _stream())  # fmt: skip
+
+
+MEMORY_MAX_KEY_DIM = 512  # a lane keeps at most 32 rows of a column of the state beside the normaliser's
+
+
+def memory_prepare(proj, q_off, k_off, v_off, i_off, f_off, num_heads, dim, vdim, i_bias, f_bias, cap, qkv, i_log, f_log) -> None:
+    """What a matrix memory's scan reads, in fp32: qkv [T, 2 H dim + H vdim] = the queries times dim^(-1/2), the keys and
+    the values out of proj [T, ld]; i_log = cap tanh((proj[:, i_off + h] + i_bias[h]) / cap) and f_log = logsigmoid(cap
+    tanh((proj[:, f_off + h] + f_bias[h]) / cap)), both [T, H]."""
+    _check(proj, "proj", (F32, BF16), (None, None))
+    T, ld = proj.shape
+    H = num_heads
+    if min(q_off, k_off, v_off, i_off, f_off) < 0 or max(q_off, k_off) + H * dim > ld or v_off + H * vdim > ld \
+            or max(i_off, f_off) + H > ld:  # fmt: skip
+        raise KernelError("memory_prepare: columns outside the projection")
+    _check(i_bias, "i_bias", F32, (H,))
+    _check(f_bias, "f_bias", F32, (H,))
+    _check(qkv, "qkv", F32, (T, 2 * H * dim + H * vdim))
+    _check(i_log, "i_log", F32, (T, H))
+    _check(f_log, "f_log", F32, (T, H))
+    call("as_memory_prepare", _ptr(proj), _DT[proj.dtype], ld, q_off, k_off, v_off, i_off, f_off, H, dim, vdim,
+         _ptr(i_bias), _ptr(f_bias), float(cap), _ptr(qkv), _ptr(i_log), _ptr(f_log), T, _stream())  # fmt: skip
+
+
+def memory_scan(qkv, num_heads, dim, vdim, i_log, f_log, state, norm_state, max_state, step_rows, out, writes=True, slices=0) -> None:
+    """A matrix memory with exponential gates over each row's tokens, per head, with a running maximum m (0 at a
+    sequence's start): m' = max(f + m, i); S' = e^(f + m - m') S + e^(i - m') k v^T; n' likewise with k;
+    out = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6).  state [slots, H, dim, vdim], norm_state [slots, H, dim], max_state
+    [slots, H], all fp32; qkv, i_log, f_log as `memory_prepare` left them; out fp32 [T, H, vdim]."""
+    _check(qkv, "qkv", F32, (None, None))
+    T, C = qkv.shape
+    H = num_heads
+    if C != 2 * H * dim + H * vdim or dim > MEMORY_MAX_KEY_DIM:
+        raise KernelError(f"memory_scan: {C} channels are not {H} x (2 x {dim} + {vdim}), or keys wider than {MEMORY_MAX_KEY_DIM}")
+    _check(i_log, "i_log", F32, (T, H))
+    _check(f_log, "f_log", F32, (T, H))
+    _check(state, "state", F32, (None, H, dim, vdim))
+    slots = state.shape[0]
+    _check(norm_state, "norm_state", F32, (slots, H, dim))
+    _check(max_state, "max_state", F32, (slots, H))
+    _check(out, "out", F32, (T, H, vdim))
+    R = _check_rows((None, *step_rows[1:]), 0)
+    _, row_first, row_len, row_start, row_slots = step_rows
+    call("as_memory_scan", _ptr(qkv), C, dim, H, vdim, _ptr(i_log), _ptr(f_log), _ptr(state), _ptr(norm_state),
+         _ptr(max_state), _ptr(row_first), _ptr(row_len), _ptr(row_start), _ptr(row_slots), int(bool(writes)), _ptr(out),
+         R, int(slices), _stream())  # fmt: skip
 
 
 def rglru_gates(u, ra, ra_bias, ri, ri_bias, lam, c, a_out, x_out) -> None:
@@ -1471,13 +1650,16 @@ def moe_route_sigmoid(h, router, top: int) -> ExpertRoute:
     return moe_route_scores(h, router, top, "sigmoid")
 
 
-ROUTER_SCORES = {"sigmoid": 0, "softmax_of_chosen": 1}
+ROUTER_SCORES = {"sigmoid": 0, "softmax_of_chosen": 1, "softmax": 2}
 
 
-def moe_route_scores(h, router, top: int, score: str, bias=None) -> ExpertRoute:
+def moe_route_scores(h, router, top: int, score: str, bias=None, groups: int = 1, keep_groups: int = 1,
+                     weight_scale: float = 1.0) -> ExpertRoute:  # fmt: skip
     """Routes by a router's logits z = router h + bias in fp32 (bias fp32 [experts] or None).  score "sigmoid": the
     `top` largest sigmoid(z), weighing s / (their sum + 1e-20); "softmax_of_chosen": the `top` largest z, weighing the
-    softmax over those z alone.  The route carries `pair_weight` fp32 [T * top] for `moe_combine`."""
+    softmax over those z alone; "softmax": s = softmax(z) over all experts, the `top` largest among the experts of the
+    `keep_groups` best of `groups` equal groups of neighbours (a group scores its largest s), weighing s * weight_scale.
+    The route carries `pair_weight` fp32 [T * top] for `moe_combine`."""
     _check(h, "h", (F32, BF16), (None, None))
     T, K = h.shape
     _check(router, "router", h.dtype, (None, K))
@@ -1488,10 +1670,15 @@ def moe_route_scores(h, router, top: int, score: str, bias=None) -> ExpertRoute:
         _check(bias, "bias", F32, (experts,))
     if not 1 <= top <= experts <= MOE_MAX_EXPERTS:
         raise KernelError(f"routing chooses up to {MOE_MAX_EXPERTS} experts, not {top} of {experts}")
+    if score != "softmax" and (groups, keep_groups, weight_scale) != (1, 1, 1.0):
+        raise KernelError("groups of experts and a scale of the weights belong to the score 'softmax'")
+    if groups < 1 or experts % groups or not 1 <= keep_groups <= groups or keep_groups * (experts // groups) < top:
+        raise KernelError(f"{experts} experts in {groups} groups of which {keep_groups} are kept do not give {top} to choose")
     route = ExpertRoute(T, top, experts, h.device)
     pair_expert = torch.empty(max(T * top, 1), dtype=I32, device=h.device)
     route.pair_weight = torch.empty(max(T * top, 1), dtype=F32, device=h.device)
-    call("as_moe_route_scores", _ptr(h), _ptr(router), _ptr(bias), ROUTER_SCORES[score], _DT[h.dtype], K, experts, top, T,
+    call("as_moe_route_scores", _ptr(h), _ptr(router), _ptr(bias), ROUTER_SCORES[score], int(groups), int(keep_groups),
+         float(weight_scale), _DT[h.dtype], K, experts, top, T,
          _ptr(pair_expert), _ptr(route.pair_weight), _stream())  # fmt: skip
     call("as_moe_route_table", 0, _ptr(pair_expert), 0, top, experts, T, _ptr(route.order), _ptr(route.tiles),
          _ptr(route.counts), route.max_tiles, _stream())  # fmt: skip

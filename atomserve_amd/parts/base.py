@@ -150,6 +150,15 @@ class GatedDelta:
         return GatedDelta(self.y, self.gate, self.gate_off, self.bias, self.mult * factor)
 
 
+class StreamsDelta:
+    """A part's output `y` [T, hidden] still to be written into several residual streams: every stream r becomes
+    sum_s mix[s, r] x_s + mult out[r] y (mix fp32 [S, S] or None for the identity, out fp32 [S]).  The kernel that reads
+    the streams for the next part does the write on its way."""
+
+    def __init__(self, y, mix, out, mult: float):
+        self.y, self.mix, self.out, self.mult = y, mix, out, mult
+
+
 class Mixer(Part):
     # Two optional shortcuts an arrangement may take with a part that declares them:
     # takes_pending_norm: `h` may arrive as a PendingNorm instead of normalised rows;
@@ -266,5 +275,5 @@ def build(family: str, spec: Any, env: BuildEnv):
 
 def _load_builtin() -> None:
     from atomserve_amd.parts import (  # noqa: F401
-        attention, block, experts, latent_attention, linear_attention, mlp, norm, recurrent, rope,
+        attention, block, experts, joined, latent_attention, linear_attention, mlp, norm, recurrent, rope,
     )

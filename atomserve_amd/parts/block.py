@@ -5,6 +5,8 @@
 "gated_prenorm": x += m g1(h) * mixer(h), h = norm(x);  x += m g2(h) * ffn(h), h = norm(x), with sigmoid gates g
 "depth_prenorm": "prenorm" whose mixer may read a token-shifted norm, and whose result may be averaged with the
               results of all layers before it
+"streams_prenorm": "prenorm" over several residual streams that a sublayer reads as one weighted sum and writes
+              through a mixing matrix
 
 The residual stream `x` is fp32 in both precisions.  A part's output is not added at
 once: it travels as the pending `delta` to the next norm, whose kernel adds it into
@@ -23,6 +25,7 @@ from atomserve_amd.parts.base import (
     Part,
     PendingNorm,
     StateCacheRequest,
+    StreamsDelta,
     WeightDecl,
     build,
     register,
@@ -238,3 +241,105 @@ class DepthPreNormBlock(Arrangement):
 
 
 register("arrangement", "depth_prenorm", DepthPreNormBlock)
+
+
+class StreamCoefficients(Part):
+    """What the sublayers of a layer over several streams read and write them with: per sublayer q (1: mixer, 2:
+    feed-forward) `hc<q>.in` [S], `hc<q>.mix` [S, S] (indexed [from, to]) and `hc<q>.out` [S]; fp32 once bound."""
+
+    capturable = True
+
+    def weight_decls(self) -> dict:
+        s, decls = self.spec, {}
+        for q in (1, 2) if s.ffn is not None else (1,):
+            decls[f"hc{q}.in"] = WeightDecl((s.streams,), role="vector")
+            decls[f"hc{q}.mix"] = WeightDecl((s.streams, s.streams), role="vector")
+            decls[f"hc{q}.out"] = WeightDecl((s.streams,), role="vector")
+        return decls
+
+    def bind(self, tensors: dict) -> None:
+        super().bind({name: t.float().contiguous() for name, t in tensors.items()})
+
+
+class StreamsPreNormBlock(Arrangement):
+    """Pre-norm sublayers over S residual streams x_1 .. x_S (fp32 [T, S, hidden], kept in the step's shared results):
+
+        u = sum_s a[s] x_s;  y = part(norm(u));  x_r <- sum_s M[s, r] x_s + m c[r] y      (m = spec.residual_scale)
+
+    with a, M, c of the sublayer's own.  The layer marked `streams_first` makes the streams, all equal to the stream it
+    is handed; the one marked `streams_last` leaves their sum as that stream again.  A part's output is not written at
+    once: it travels as a pending `StreamsDelta` to the kernel that reads the streams for the next part
+    (`ops.streams_step`), which writes, reads and norms in one pass.  spec.streams 0: one stream and a = M = c = 1, the
+    plain `x += m y`."""
+
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        self.mixer_norm = build("norm", spec.mixer_norm, env)
+        self.mixer = build("mixer", spec.mixer, env)
+        self.ffn_norm = self.ffn = None
+        if spec.ffn is not None:
+            self.ffn_norm = build("norm", spec.ffn_norm, env)
+            self.ffn = build("feed_forward", spec.ffn, env)
+        for norm in (self.mixer_norm, self.ffn_norm):
+            if norm is not None and norm.spec.kind != "rmsnorm":
+                raise ValueError(f"the kernel that reads several streams norms by 'rmsnorm', not by {norm.spec.kind!r}")
+        if not 0 <= spec.streams <= ops.STREAMS_MAX:
+            raise ValueError(f"0 to {ops.STREAMS_MAX} streams, not {spec.streams}")
+        self.coefficients = StreamCoefficients(spec, env) if spec.streams else None
+        self.ones = None
+
+    def parts(self) -> dict:
+        parts = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        if self.ffn is not None:
+            parts.update(ffn_norm=self.ffn_norm, ffn=self.ffn)
+        if self.coefficients is not None:
+            parts["streams"] = self.coefficients
+        return parts
+
+    def first_norm(self):
+        return None  # nothing is left pending inside a product for this layer
+
+    def _coefficients(self, q: int, device):
+        """(in, mix, out) of sublayer q."""
+        c = self.coefficients
+        if c is None:
+            if self.ones is None:
+                self.ones = torch.ones(1, dtype=torch.float32, device=device)
+            return self.ones, None, self.ones
+        return getattr(c, f"hc{q}_in"), getattr(c, f"hc{q}_mix"), getattr(c, f"hc{q}_out")
+
+    def forward(self, x, delta, step, cache, next_norm=None):
+        s, env = self.spec, self.env
+        T, n = x.shape
+        first = None
+        if s.streams_first:
+            if delta is not None:
+                raise ValueError("the first of the layers over several streams starts from a complete stream")
+            xs = step.shared["streams"] = torch.empty((T, max(s.streams, 1), n), dtype=torch.float32, device=x.device)
+            first = x
+        else:
+            xs = step.shared.get("streams")
+            if xs is None or xs.shape != (T, max(s.streams, 1), n) or not isinstance(delta, StreamsDelta):
+                raise ValueError("the layers over several streams run in order, from the first, within one step")
+        pending = delta
+        for q, norm, part in ((1, self.mixer_norm, self.mixer), (2, self.ffn_norm, self.ffn)):
+            if part is None:
+                continue
+            a, mix, c = self._coefficients(q, x.device)
+            h = torch.empty((T, n), dtype=env.dtype, device=x.device)
+            if pending is None:
+                ops.streams_step(xs, first=first, in_c=a, gain=norm.gain_f32, eps=norm.spec.eps, normed=h)
+            else:
+                ops.streams_step(xs, y=pending.y, mix=pending.mix, out_c=pending.out, mult=pending.mult, in_c=a,
+                                 gain=norm.gain_f32, eps=norm.spec.eps, normed=h)  # fmt: skip
+            y = part.forward(h, step, cache) if q == 1 else part.forward(h, step)
+            if not isinstance(y, torch.Tensor):
+                raise ValueError("a part of a layer over several streams returns its output, nothing pending of its own")
+            pending = StreamsDelta(y, mix, c, s.residual_scale)
+        if not s.streams_last:
+            return pending
+        ops.streams_step(xs, y=pending.y, mix=pending.mix, out_c=pending.out, mult=pending.mult, total=x)
+        return None
+
+
+register("arrangement", "streams_prenorm", StreamsPreNormBlock)

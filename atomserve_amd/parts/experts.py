@@ -145,6 +145,8 @@ class GatedRoutedExperts(FeedForward):
     """Gated experts chosen by a router with a bias:
 
         z = R h + b in fp32; a token's `top` experts are those with the largest z, weighing the softmax over those z alone
+        (spec.score "softmax_of_chosen"), or those with the largest softmax(z) among the experts of the best groups, weighing
+        that softmax times a factor ("softmax", `GatedRoutedExpertsSpec`)
         expert e: down_e(act(gate_e h, up_e h)), act the gated activation of the spec with its limit
         with spec.shared_size one more such expert (with a limit of its own) runs for every token and is added
 
@@ -198,7 +200,8 @@ class GatedRoutedExperts(FeedForward):
         s, env = self.spec, self.env
         T, dev = h.shape[0], h.device
         clamped = s.activation == "clamped_swish"
-        route = ops.moe_route_scores(h, self.router_weight, s.top, s.score, self.router_bias)
+        route = ops.moe_route_scores(h, self.router_weight, s.top, s.score, self.router_bias, s.groups, s.keep_groups,
+                                     s.weight_scale)  # fmt: skip
         pairs = T * s.top
         act = torch.empty((pairs, s.intermediate_size), dtype=env.dtype, device=dev)
         ops.moe_gemm(h, self.gate_up_weight, route, act, gated=True, per_token=True, limit=s.limit if clamped else 0.0)

@@ -37,6 +37,8 @@ class RMSNorm(Norm):
 
     def bind(self, tensors: dict) -> None:
         super().bind(tensors)
+        if self.spec.offset:  # a gain stored around zero: the sum is made once, in 32 bits, and stays so
+            self.weight = (self.weight.float() + float(self.spec.offset)).contiguous()
         self.gain_f32 = self.weight.float()  # what the fused product reads (exact: bf16 widens)
 
     def absorb(self, a, w, x):

@@ -19,6 +19,7 @@ class NormSpec:
     size: int
     eps: float
     groups: int = 1
+    offset: float = 0.0  # added to the stored gain (1.0: a gain stored around zero); the sum is kept in 32 bits
 
 
 @dataclass(frozen=True)
@@ -46,6 +47,20 @@ class ScaledRotarySpec:
     original: float
     fast: float
     slow: float
+
+
+@dataclass(frozen=True)
+class NeighbourRotarySpec:
+    """Rotary position encoding of a head's first `rotary_dim` coordinates whose pairs are neighbours, (2i, 2i + 1).
+    kind "rope_neighbours".  With `factor` > 0 the frequencies are stretched as `ScaledRotarySpec` says."""
+
+    kind: str
+    rotary_dim: int
+    theta: float
+    factor: float = 0.0
+    original: float = 0.0
+    fast: float = 0.0
+    slow: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -204,6 +219,75 @@ class SideBySideSpec:
 
 
 @dataclass(frozen=True)
+class SoftmaxCoreSpec:
+    """A grouped-query causal softmax attention as one of the cores of a "joined" mixer: keys and queries `key_dim`
+    wide, values `value_dim`.  bias: q, k and v have biases.  whole_norm_eps > 0: q and k are RMS-normed over their
+    whole projection (all heads at once) with gains of that size.  position: a rotation of q and k, or None.
+    value_mix "first": the core's values (of the step's tokens) are kept for later layers under `value_mix_key`;
+    "later": its values become (1 - lam) v + lam v_first before they are cached, lam a scalar of its own.
+    out_gate: the concatenated heads are multiplied by sigmoid of a projection of the input."""
+
+    kind: str  # "softmax_core"
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    bias: bool = False
+    whole_norm_eps: float = 0.0
+    position: Any = None
+    value_mix: str = "none"
+    value_mix_key: str = "values"
+    out_gate: bool = False
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """A matrix memory with exponential gates, per head: a state S [key_dim, value_dim], a normaliser n [key_dim] and
+    a running maximum m (0 at the start) of the gates' logarithms i = cap tanh(. / cap) and f = logsigmoid(cap tanh(. / cap)):
+    m' = max(f + m, i); S' = e^(f + m - m') S + e^(i - m') k v^T, n' likewise with k; o = S'^T q / (max(|n' . q|, e^(-m')) +
+    1e-6) with q times key_dim^(-1/2).  Every head's o over its root mean square, the heads times a gain [heads x
+    value_dim] and sigmoid of a projection of the input.  One of the cores of a "joined" mixer."""
+
+    kind: str  # "matrix_memory"
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    gate_cap: float
+    out_norm_eps: float
+
+
+@dataclass(frozen=True)
+class JoinedMixerSpec:
+    """Several cores that read the same input; one input product makes what all of them need and one output product
+    takes scales[c] * core c's result side by side, so the weighted sum of the cores is the product's own sum."""
+
+    kind: str  # "joined"
+    hidden_size: int
+    cores: tuple
+    scales: tuple
+
+
+@dataclass(frozen=True)
+class ChannelDeltaRuleSpec:
+    """The gated delta rule of `DeltaRuleSpec` with a decay per head and key channel, g = exp(-exp(A_h) softplus(W_2
+    (W_1 h) + b)) laid out heads x key_dim and acting on the rows of S; the output is normed per head (a gain
+    [value_dim] shared by the heads) and times sigmoid(G_2 (G_1 h)).  decay_rank and gate_rank: rows of W_1 and G_1."""
+
+    kind: str  # "channel_delta_rule"
+    hidden_size: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    conv: ShortConvSpec
+    decay_rank: int
+    gate_rank: int
+    out_norm_eps: float
+    unit_eps: float = 1e-6
+
+
+@dataclass(frozen=True)
 class TableExpertsSpec:
     """Gated feed-forward experts of which every token uses `top`, named by a table indexed with the
     token id; each chosen expert weighs 1 / top."""
@@ -238,7 +322,10 @@ class RoutedExpertsSpec:
 @dataclass(frozen=True)
 class GatedRoutedExpertsSpec:
     """Gated experts chosen by a router: z = router h + bias in fp32, the `top` largest z are chosen and weigh the
-    softmax over the chosen z alone (`score` "softmax_of_chosen").  An expert is down(act(gate h, up h)) with the
+    softmax over the chosen z alone (`score` "softmax_of_chosen").  `score` "softmax": s = softmax(z) over all
+    experts; the experts form `groups` equal groups of neighbours, a group scores its largest s, and the `top`
+    largest s among the experts of the `keep_groups` best groups are chosen; they weigh s * weight_scale, not
+    renormalised.  An expert is down(act(gate h, up h)) with the
     activation of `GatedMLPSpec` and `limit`.  shared_size > 0: one more such expert (with `shared_limit`) runs for
     every token and is added."""
 
@@ -253,6 +340,9 @@ class GatedRoutedExpertsSpec:
     router_bias: bool = True
     shared_size: int = 0
     shared_limit: float = 0.0
+    groups: int = 1
+    keep_groups: int = 1
+    weight_scale: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -267,7 +357,11 @@ class BlockSpec:
     reads is h_t + (h_(t-1) - h_t) * shift, h the mixer's norm of the stream (zeros before a sequence's first token;
     the last h is part of a request's state).  depth_slots > 0: the layer's result is kept as number depth_index + 1
     of depth_slots results (number 0 is what the embedding gave), and the stream goes on as their weighted sum with
-    depth_index + 2 weights of the layer's own."""
+    depth_index + 2 weights of the layer's own.
+    arrangement "streams_prenorm": the stream is `streams` copies x_1 .. x_s (all what the embedding gave before the
+    layer marked streams_first); a sublayer reads u = sum_s a[s] x_s through its norm and writes x_t <- sum_s M[s, t]
+    x_s + residual_scale c[t] y with a, M, c of its own; the layer marked streams_last leaves their sum as the
+    stream.  streams 0: one stream with a = M = c = 1, that is x += residual_scale y."""
 
     arrangement: str
     mixer: Any
@@ -278,6 +372,9 @@ class BlockSpec:
     token_shift: bool = False
     depth_index: int = 0
     depth_slots: int = 0
+    streams: int = 0
+    streams_first: bool = False
+    streams_last: bool = False
 
 
 @dataclass(frozen=True)

@@ -217,5 +217,98 @@ class SideBySide(Mixer):
         return y
 
 
+class ChannelDeltaRule(Mixer):
+    """The gated delta rule with a decay per head and key channel (`ChannelDeltaRuleSpec`), per head h:
+        S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+    q, k, v = silu(conv(W h)), q and k unit vectors (q also times key_dim^(-1/2)), beta = sigmoid(W_b h),
+    g = exp(-exp(A_log[h]) softplus(W_a2 (W_a1 h) + dt_bias)) laid out heads x key_dim; the output is
+    o / rms(o) * weight * sigmoid(W_g2 (W_g1 h)) through W_o.  Three products read: `in` (q, k, v, beta), `low` (the first
+    steps W_a1 and W_g1 stacked) and `expand`, which is W_a2 and W_g2 on the diagonal of one matrix, so that the two
+    second steps are one product of `low`'s result."""
+
+    capturable = True
+
+    def __init__(self, spec, env):
+        super().__init__(spec, env)
+        s = spec
+        if s.num_heads % s.num_kv_heads:
+            raise ValueError(f"{s.num_heads} value heads do not divide over {s.num_kv_heads} key heads")
+        if not 1 <= s.conv.taps <= ops.CONV_MAX_TAPS:
+            raise ValueError(f"a short convolution has 1 to {ops.CONV_MAX_TAPS} taps, not {s.conv.taps}")
+        if s.decay_rank < 1 or s.gate_rank < 1:
+            raise ValueError("the two-step projections of the decay and of the output gate have ranks of at least 1")
+        qk, v = s.num_kv_heads * s.key_dim, s.num_heads * s.value_dim
+        self.channels = 2 * qk + v  # what passes the convolution: q, k, v
+        self.beta_off = self.channels
+        self.in_rows = self.beta_off + s.num_heads
+        self.step_cols = s.num_heads * s.key_dim  # columns of the expanded product: step sizes, then the gate
+        self.wide_cols = self.step_cols + v
+
+    def weight_decls(self) -> dict:
+        s = self.spec
+        return {
+            "in.weight": WeightDecl((self.in_rows, s.hidden_size)),
+            "low.weight": WeightDecl((s.decay_rank + s.gate_rank, s.hidden_size)),
+            "decay_up.weight": WeightDecl((self.step_cols, s.decay_rank)),
+            "gate_up.weight": WeightDecl((s.num_heads * s.value_dim, s.gate_rank)),
+            "conv.weight": WeightDecl((self.channels, s.conv.taps), role="vector"),
+            "a_log": WeightDecl((s.num_heads,), role="vector"),
+            "dt_bias": WeightDecl((self.step_cols,), role="vector"),
+            "out_norm.weight": WeightDecl((s.value_dim,), role="vector"),
+            "out.weight": WeightDecl((s.hidden_size, s.num_heads * s.value_dim)),
+        }
+
+    def bind(self, tensors: dict) -> None:
+        super().bind(tensors)
+        s = self.spec
+        for name in ("conv_weight", "a_log", "dt_bias", "out_norm_weight"):
+            setattr(self, name, getattr(self, name).float().contiguous())
+        expand = torch.zeros((self.wide_cols, s.decay_rank + s.gate_rank), dtype=self.in_weight.dtype, device=self.in_weight.device)
+        expand[: self.step_cols, : s.decay_rank] = self.decay_up_weight
+        expand[self.step_cols :, s.decay_rank :] = self.gate_up_weight
+        del self.decay_up_weight, self.gate_up_weight
+        self.inp = ops.Streamed(self.in_weight, self.env.stream_copies)
+        self.low = ops.Streamed(self.low_weight, self.env.stream_copies)
+        self.expand = ops.Streamed(expand, self.env.stream_copies)
+        self.out = ops.Streamed(self.out_weight, self.env.stream_copies)
+
+    def streamed(self) -> list:
+        return [self.inp, self.low, self.expand, self.out]
+
+    def cache_request(self):
+        s = self.spec
+        asked = {"state": StateCacheRequest((s.num_heads, s.key_dim, s.value_dim), torch.float32)}
+        if s.conv.taps > 1:
+            asked["conv"] = StateCacheRequest((s.conv.taps - 1, self.channels), torch.float32)
+        return asked
+
+    def forward(self, h, step, cache):
+        s, env = self.spec, self.env
+        T, dev = h.shape[0], h.device
+        H, G = s.num_heads, s.num_kv_heads
+        proj = torch.empty((T, self.in_rows), dtype=env.dtype, device=dev)
+        ops.gemm(h, self.inp, proj, env.products)
+        low = torch.empty((T, s.decay_rank + s.gate_rank), dtype=env.dtype, device=dev)
+        ops.gemm(h, self.low, low, env.products)
+        wide = torch.empty((T, self.wide_cols), dtype=env.dtype, device=dev)
+        ops.gemm(low, self.expand, wide, env.products)
+        rows = _step_rows(step)
+        state = cache["state"]
+        history = cache["conv"].state if "conv" in cache else torch.empty((1, 0, self.channels), dtype=torch.float32, device=dev)
+        qkv = torch.empty((T, self.channels), dtype=torch.float32, device=dev)
+        ops.short_conv(proj, 0, self.conv_weight, history, rows, qkv, silu=True, writes=state.writes)
+        beta = torch.empty((T, H), dtype=torch.float32, device=dev)
+        chan = torch.empty((T, H, s.key_dim), dtype=torch.float32, device=dev)
+        ops.delta_prepare_channels(qkv, G, s.key_dim, H, proj, self.beta_off, wide, 0, self.a_log, self.dt_bias, beta, chan)
+        o = torch.empty((T, H, s.value_dim), dtype=torch.float32, device=dev)
+        ops.delta_scan_channels(qkv, G, s.key_dim, H, s.value_dim, beta, chan, state.state, rows, o, writes=state.writes)
+        act = torch.empty((T, H * s.value_dim), dtype=env.dtype, device=dev)
+        ops.delta_finish(o, self.out_norm_weight, s.out_norm_eps, wide, self.step_cols, act, gate="sigmoid")
+        y = torch.empty((T, s.hidden_size), dtype=env.dtype, device=dev)
+        ops.gemm(act, self.out, y, env.products)
+        return y
+
+
 register("mixer", "delta_rule", DeltaRule)
+register("mixer", "channel_delta_rule", ChannelDeltaRule)
 register("mixer", "side_by_side", SideBySide)

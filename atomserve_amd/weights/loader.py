@@ -156,6 +156,22 @@ class SafetensorsSource:
         return self.where[name].get_tensor(name)
 
 
+def checkpoint_shapes_of(model_dir: str):
+    """name -> shape of a tensor in the folder's *.safetensors files (None for a name they lack), read from the
+    files' headers alone: an 8-byte little-endian length, that many bytes of JSON (name -> dtype, shape, offsets)."""
+    import struct
+
+    shapes = {}
+    for path in sorted(glob.glob(os.path.join(model_dir, "*.safetensors"))):
+        with open(path, "rb") as f:
+            (length,) = struct.unpack("<Q", f.read(8))
+            header = json.loads(f.read(length))
+        for name, entry in header.items():
+            if name != "__metadata__":
+                shapes[name] = tuple(entry["shape"])
+    return shapes.get
+
+
 def _storage_dtype(role: str, stored: torch.dtype, compute: torch.dtype) -> torch.dtype:
     if role == "table_int":
         return torch.int32
@@ -195,6 +211,8 @@ def bind_checkpoint(model, arch, config, source, where: str = "") -> dict:
         if recipes[target].new_axis:
             made = (len(shapes), *shapes[0])
             alike = all(sh == shapes[0] for sh in shapes)
+        elif len(shapes) == 1:  # one piece as it is (also a scalar, which has no rows to stack)
+            made, alike = shapes[0], True
         else:
             made = (sum(sh[0] for sh in shapes), *shapes[0][1:])
             alike = all(sh[1:] == shapes[0][1:] for sh in shapes)
