@@ -7,7 +7,7 @@
 // part's product left it) and the normed rows (the next product's input) are in the compute dtype.
 #include "common.h"
 
-#define STREAMS_MAX 8
+#define STREAMS_MAX 16
 #define STREAMS_KEEP 8  // columns of a row that a thread keeps between the two passes of the norm
 
 // first:    the streams do not exist yet: all of them are x0 [T, n] (what the embedding gave)

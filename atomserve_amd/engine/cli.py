@@ -178,6 +178,10 @@ def main(argv=None) -> int:
             raw = json.load(f)
         arch = architecture_for(raw)
         config = arch.parse_config(raw)
+        if arch.complete is not None and args.random_weights is None:  # sizes that only the tensors' shapes tell
+            from atomserve_amd.weights.loader import checkpoint_shapes_of
+
+            config = arch.complete(config, checkpoint_shapes_of(model_dir))
         print(f"Loading {args.model} ({args.dtype}, {arch.name}) ...", file=sys.stderr, flush=True)
         model = DecoderModel(arch.build_plan(config), dtype, "cuda:0", stream_copies=not args.no_stream_copies)
         if args.random_weights is not None:

@@ -1130,7 +1130,7 @@ def whole_norm_store(proj, q_off, k_off, v_off, num_heads, num_kv_heads, dim, vd
          _ptr(v_pages) if store_kv else 0, bs, int(bool(store_kv)), T, _stream())  # fmt: skip
 
 
-STREAMS_MAX = 8
+STREAMS_MAX = 16
 
 
 def streams_step(xs, first=None, y=None, mix=None, out_c=None, mult: float = 1.0, in_c=None, gain=None, eps: float = 0.0,

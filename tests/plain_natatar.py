@@ -312,3 +312,8 @@ def forward(raw, W, tokens, bf16=False, dtype=F, layers_out=None):
             layers_out.append(xs.sum(dim=0))
     x = offset_norm(xs.sum(dim=0), W["final.norm"], eps)
     return rnd(x, bf16) @ W["embed"].t()
+
+
+def logits(raw, W, ids, rounded=False):
+    """Logits [T, vocab] in float32: exact (float64 inside), or with bfloat16 activations."""
+    return forward(raw, W, ids, bf16=rounded).float()
