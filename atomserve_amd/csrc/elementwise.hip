@@ -792,8 +792,8 @@ __global__ void sigmoid_gate_heads_kernel(const T* __restrict__ heads, int H, in
     const size_t t = idx / per;
     const int c = (int)(idx % per), h = c / vdim, j = c % vdim;
     const float v = to_f32(heads[(t * H + h) * Dp + j]);
-    const float g = gate ? 1.0f / (1.0f + expf(-to_f32(gate[t * ld_gate + gate_off + c]))) : 1.0f;  // no gate: the heads, scaled
-    out[t * ld_out + out_off + c] = from_f32<T>(scale * v * g);
+    // no gate: the heads, scaled
+    out[t * ld_out + out_off + c] = from_f32<T>(gate ? scale * v / (1.0f + expf(-to_f32(gate[t * ld_gate + gate_off + c]))) : scale * v);
   }
 }
 
