@@ -121,6 +121,10 @@ class SoftmaxCore:
                              pages.slots, q, pages.k_pages, pages.v_pages, store_kv=pages.writes, biases=self.biases,
                              gains=self.gains, eps=s.whole_norm_eps, cos_sin=cos_sin, v_keep=v_keep, v_mode=v_mode,
                              lam=self.lam)  # fmt: skip
+        if not s.out_gate and scale == 1.0 and Dp == s.value_dim and out_off == 0 and act.shape[1] == self.out_cols:
+            # the core alone, its heads as wide as they are laid out: the attention writes the output product's input itself
+            attend(q, act.view(T, H, Dp), step, pages, s.scale, 0, (SHORT_ROW, TILE_Q))
+            return
         heads = torch.empty((T, H, Dp), dtype=env.dtype, device=dev)
         attend(q, heads, step, pages, s.scale, 0, (SHORT_ROW, TILE_Q))
         ops.sigmoid_gate_heads(heads, s.value_dim, proj if s.out_gate else None, off + self.gate_off, scale, act, out_off)

@@ -5,6 +5,7 @@
     python bench.py --design dozusun [--widths 1024,2048,4096]   (Dozusun layers beside Qwen3 layers of equal size)
     python bench.py --design koravik [--widths 1024,2048,4096]   (Koravik layers beside Qwen3 layers of equal size)
     python bench.py --design mumizen [--widths 1024,2048,4096]   (Mumizen layers beside Qwen3 layers of equal size)
+    python bench.py --design natatar [--widths 1024,2048,4096]   (Natatar layers beside Dozusun and Qwen3 layers of equal size)
 
 A step is one decode step of the engine (scheduler, one pass over the GPU, sampling).
 Prints ONE JSON line: decoded tokens per second at batch 8 with 2,048-token contexts,
@@ -77,7 +78,7 @@ def parse_args():
                         "(half of them share their first 32), chunks of 512, 128 tokens decoded each, through the "
                         "scheduler from submission to the last token")  # fmt: skip
     p.add_argument("--chunk-budget", type=int, default=512, help="token budget of a step in the mixed workload")
-    p.add_argument("--design", choices=["qwen3", "dozusun", "koravik", "mumizen"], default="qwen3",
+    p.add_argument("--design", choices=["qwen3", "dozusun", "koravik", "mumizen", "natatar"], default="qwen3",
                    help="dozusun: prefill and decode throughput of random-weight Dozusun layers (an attention beside a "
                         "gated linear recurrence, gated delta rules, dense and table-routed feed-forwards) at a few "
                         "widths, beside Qwen3 layers of the same width, heads, depth and vocabulary; koravik: the same "
@@ -236,12 +237,37 @@ def mumizen_config(width: int, layers: int, vocab: int):
                                     "norm": {"eps": 1e-6, "groups": 4}, "layers": made})  # fmt: skip
 
 
+def natatar_config(width: int, layers: int, vocab: int):
+    """Layers as a model of this design of that width would have them: four streams; heads of 128 everywhere, a kv
+    head to four query heads in the attentions; the delta rule with a key head to two value heads, four taps and
+    two-step projections of rank 64; the rotary attention (64 of a head's 128 coordinates turned, stretched
+    frequencies) beside a matrix memory of half as many heads; every feed-forward 16 experts of three quarters of the
+    width, two to a token out of the two best of four groups; the kinds of layers in turn: delta rule, attention,
+    attention beside memory, attention (the attentions mix their values with the first one's)."""
+    from atomserve_amd.config.model_config import NatatarConfig
+
+    heads = width // 128
+    kv = max(1, heads // 4)
+    attention = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128**-0.5, "v_mix": True}
+    delta = {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 64, "gate_rank": 64}
+    left = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128**-0.5,
+            "rot": {"dims": 64, "base": 1e6, "scaling": {"factor": 16.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}  # fmt: skip
+    side = {"left": left, "right": {"heads": max(1, heads // 2), "dim": 128, "vdim": 128, "gate_cap": 15.0}, "left_scale": 0.8,
+            "right_scale": 0.5}  # fmt: skip
+    mlp = {"kind": "moe", "expert": {"ff": 3 * width // 4},
+           "router": {"experts": 16, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}}  # fmt: skip
+    kinds = [("channel_delta", delta), ("attention", attention), ("parallel", side), ("attention", attention)]
+    return NatatarConfig.from_dict({"architecture": "Natatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+                                    "residual_mult": 0.7, "embedding": {"scale": 8.0}, "streams": 4,
+                                    "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": mlp} for i in range(layers)]})  # fmt: skip
+
+
 def design_comparison(args) -> dict:
     """Prefill of --prefill-tokens tokens and decode at batch 1 and --batch with --context tokens of context, for
     the layers of --design and for Qwen3 layers of equal width, heads, depth and vocabulary; random weights, the
     engine's own entry point (scheduler, captured decode steps, sampling)."""
     design = args.design
-    make = {"dozusun": dozusun_config, "koravik": koravik_config, "mumizen": mumizen_config}[design]
+    make = {"dozusun": dozusun_config, "koravik": koravik_config, "mumizen": mumizen_config, "natatar": natatar_config}[design]
     import torch
 
     from atomserve_amd.config import EngineConfig, Qwen3Config
@@ -308,6 +334,8 @@ def design_comparison(args) -> dict:
                            num_heads=heads, num_kv_heads=max(1, heads // 4), head_dim=128, rms_norm_eps=1e-6,
                            rope_theta=1e6, tie_word_embeddings=False, max_position_embeddings=40960)  # fmt: skip
         sizes[str(width)] = {design: measure(make(width, layers, vocab)), "qwen3": measure(qwen)}
+        if design == "natatar":  # its closest relative among the designs: a delta rule, an attention beside a recurrence, experts
+            sizes[str(width)]["dozusun"] = measure(dozusun_config(width, layers, vocab))
         print(f"width {width}: {json.dumps(sizes[str(width)])}", file=sys.stderr, flush=True)
     widest = sizes[max(sizes, key=int)]
     return {
@@ -362,7 +390,7 @@ def main() -> int:
     from atomserve_amd.weights.loader import DictSource, bind_checkpoint
     from atomserve_amd.weights.random_init import random_checkpoint
 
-    if args.design in ("dozusun", "koravik", "mumizen"):
+    if args.design in ("dozusun", "koravik", "mumizen", "natatar"):
         print(json.dumps(design_comparison(args)))
         return 0
     device = "cuda:0"
