@@ -695,6 +695,8 @@ __global__ __launch_bounds__(256) void whole_norm_store_kernel(
     const float* __restrict__ qw, const float* __restrict__ kw, float eps, const float2* __restrict__ cs, int R,
     float* __restrict__ v_keep, int v_mode, float lam, const int* __restrict__ slots, T* __restrict__ q_out,
     T* __restrict__ k_pages, T* __restrict__ v_pages, int bs, int store) {
+  // blockIdx.y: one of gridDim.y workgroups that share a token's heads (query, key and value heads in one list, dealt
+  // out in turn); every one of them takes the root mean squares over the whole projections for itself.
   __shared__ float red[17];
   const int t = blockIdx.x;
   const T* row = proj + (size_t)t * ld;
@@ -715,15 +717,17 @@ __global__ __launch_bounds__(256) void whole_norm_store_kernel(
   }
   const int half = cs ? R / 2 : 0;
   const int slot = (store && slots) ? slots[t] : -1;
-  // queries, then keys: coordinate d of head hh, with its partner if it turns
-  for (int which = 0; which < 2; ++which) {
-    const int heads = which ? KV : H, off = which ? k_off : q_off;
-    const float* bias = which ? k_bias : q_bias;
-    const float* w = which ? kw : qw;
-    const float inv = which ? inv_k : inv_q;
-    if (which && slot < 0) break;
-    for (int idx = threadIdx.x; idx < heads * Dp; idx += blockDim.x) {
-      const int hh = idx / Dp, d = idx - hh * Dp;
+  const int all = H + 2 * KV, share = (all - (int)blockIdx.y + (int)gridDim.y - 1) / (int)gridDim.y;  // heads of this workgroup
+  for (int idx = threadIdx.x; idx < share * Dp; idx += blockDim.x) {
+    const int head = blockIdx.y + (idx / Dp) * gridDim.y, d = idx % Dp;
+    if (head < H + KV) {  // a query or a key head: coordinate d, with its partner if it turns
+      const bool is_k = head >= H;
+      const int hh = is_k ? head - H : head, off = is_k ? k_off : q_off;
+      const float* bias = is_k ? k_bias : q_bias;
+      const float* w = is_k ? kw : qw;
+      const float inv = is_k ? inv_k : inv_q;
+      if (is_k && slot < 0) continue;
+      T* dst = is_k ? k_pages + (((size_t)(slot / bs) * KV + hh) * bs + slot % bs) * Dp : q_out + ((size_t)t * H + hh) * Dp;
       auto value = [&](int dd) {
         const int c = hh * dim + dd;
         float v = to_f32(row[off + c]) + (bias ? bias[c] : 0.f);
@@ -737,22 +741,18 @@ __global__ __launch_bounds__(256) void whole_norm_store_kernel(
         const float2 a = cs[(size_t)t * half + i];
         v = d < half ? v * a.x - u * a.y : v * a.x + u * a.y;
       }
-      T* dst = which ? k_pages + (((size_t)(slot / bs) * KV + hh) * bs + slot % bs) * Dp
-                     : q_out + ((size_t)t * H + hh) * Dp;
       dst[d] = from_f32<T>(finite_or_zero(v));
+    } else {  // a value head
+      const int g = head - H - KV;
+      float v = 0.f;
+      if (d < vdim) {
+        const int c = g * vdim + d;
+        v = to_f32(row[v_off + c]) + (v_bias ? v_bias[c] : 0.f);
+        if (v_mode == 1) v_keep[(size_t)t * nv + c] = v;
+        else if (v_mode == 2) v = (1.0f - lam) * v + lam * v_keep[(size_t)t * nv + c];
+      }
+      if (slot >= 0) v_pages[((size_t)(slot / bs) * KV + g) * Dp * bs + (size_t)d * bs + slot % bs] = from_f32<T>(finite_or_zero(v));
     }
-  }
-  // values
-  for (int idx = threadIdx.x; idx < KV * Dp; idx += blockDim.x) {
-    const int g = idx / Dp, d = idx - g * Dp;
-    float v = 0.f;
-    if (d < vdim) {
-      const int c = g * vdim + d;
-      v = to_f32(row[v_off + c]) + (v_bias ? v_bias[c] : 0.f);
-      if (v_mode == 1) v_keep[(size_t)t * nv + c] = v;
-      else if (v_mode == 2) v = (1.0f - lam) * v + lam * v_keep[(size_t)t * nv + c];
-    }
-    if (slot >= 0) v_pages[((size_t)(slot / bs) * KV + g) * Dp * bs + (size_t)d * bs + slot % bs] = from_f32<T>(finite_or_zero(v));
   }
 }
 
@@ -767,12 +767,16 @@ extern "C" int as_whole_norm_store(const void* proj, int dtype, int ld, int q_of
   if (H <= 0 || KV <= 0 || dim <= 0 || vdim <= 0 || Dp < dim || Dp < vdim || bs <= 0 || ld <= 0 || (!qw) != (!kw))
     return AS_BAD_SHAPE;
   if (v_mode < 0 || v_mode > 2 || (v_mode && !v_keep)) return AS_BAD_SHAPE;
+  // few tokens (a decode step): a token's heads are dealt out over several workgroups; many: one takes them all
+  int across = num_tokens >= 256 ? 1 : (H + 2 * KV < 32 ? H + 2 * KV : 32);
+  const int threads = across > 1 && Dp <= 128 ? (Dp > 64 ? 128 : 64) : 256;
+  dim3 grid(num_tokens, across);
   if (dtype == DT_F32)
-    whole_norm_store_kernel<float><<<num_tokens, 256, 0, stream>>>(
+    whole_norm_store_kernel<float><<<grid, threads, 0, stream>>>(
         (const float*)proj, ld, q_off, k_off, v_off, H, KV, dim, vdim, Dp, q_bias, k_bias, v_bias, qw, kw, eps,
         (const float2*)cs, R, v_keep, v_mode, lam, slots, (float*)q_out, (float*)k_pages, (float*)v_pages, bs, store);
   else if (dtype == DT_BF16)
-    whole_norm_store_kernel<bf16><<<num_tokens, 256, 0, stream>>>(
+    whole_norm_store_kernel<bf16><<<grid, threads, 0, stream>>>(
         (const bf16*)proj, ld, q_off, k_off, v_off, H, KV, dim, vdim, Dp, q_bias, k_bias, v_bias, qw, kw, eps,
         (const float2*)cs, R, v_keep, v_mode, lam, slots, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages, bs, store);
   else return AS_BAD_DTYPE;

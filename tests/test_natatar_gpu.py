@@ -722,7 +722,7 @@ def test_channel_delta_rule_keeps_a_far_token():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("sizes", [(1, 40), (2, 96), (3, 256), (4, 1032), (8, 40), (3, 9000)])
+@pytest.mark.parametrize("sizes", [(1, 40), (2, 96), (3, 256), (4, 1032), (8, 40), (3, 9000), (2, 4101), (5, 16400), (16, 24)])
 def test_streams_are_written_read_and_normed_in_one_pass(sizes, dtype):
     from atomserve_amd.kernels import ops
 
