@@ -856,8 +856,8 @@ class NatatarConfig:
                 if a.rot and (a.rot[0] < 2 or a.rot[0] % 2 or a.rot[0] > a.dim or not a.rot[1] > 1):
                     raise ConfigError(f"layers[{i}]: rot.dims is even and at most dim, rot.base exceeds 1")
             if layer.type == "attention" and m.v_mix:
-                if mixed is not None and (mixed.kv_heads, mixed.vdim) != (m.kv_heads, m.vdim):
-                    raise ConfigError(f"layers[{i}]: layers that mix values have values of one shape")
+                if mixed is not None and mixed.kv_heads * mixed.vdim != m.kv_heads * m.vdim:
+                    raise ConfigError(f"layers[{i}]: layers that mix values have value projections of one size")
                 mixed = mixed or m
             if layer.type == "parallel" and min(m.right.heads, m.right.dim, m.right.vdim) < 1:
                 raise ConfigError(f"layers[{i}]: the memory's head count and sizes must be positive")

@@ -252,13 +252,13 @@ def natatar_config(width: int, layers: int, vocab: int):
     delta = {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 64, "gate_rank": 64}
     left = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128**-0.5,
             "rot": {"dims": 64, "base": 1e6, "scaling": {"factor": 16.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}  # fmt: skip
-    side = {"left": left, "right": {"heads": max(1, heads // 2), "dim": 128, "vdim": 128, "gate_cap": 15.0}, "left_scale": 0.8,
-            "right_scale": 0.5}  # fmt: skip
+    side = {"left": left, "right": {"heads": max(1, heads // 2), "dim": 128, "vdim": 128, "gate_cap": 12.0}, "left_scale": 0.6,
+            "right_scale": 0.9}  # fmt: skip
     mlp = {"kind": "moe", "expert": {"ff": 3 * width // 4},
-           "router": {"experts": 16, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}}  # fmt: skip
+           "router": {"experts": 16, "top": 2, "scale": 1.5, "groups": {"count": 4, "keep": 2}}}  # fmt: skip
     kinds = [("channel_delta", delta), ("attention", attention), ("parallel", side), ("attention", attention)]
     return NatatarConfig.from_dict({"architecture": "Natatar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
-                                    "residual_mult": 0.7, "embedding": {"scale": 8.0}, "streams": 4,
+                                    "residual_mult": 0.5, "embedding": {"scale": 8.0}, "streams": 4,
                                     "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": mlp} for i in range(layers)]})  # fmt: skip
 
 

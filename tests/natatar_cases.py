@@ -67,7 +67,7 @@ CASES = {
     "plain_sums": {
         "architecture": "Natatar", "vocab": 203, "width": 88, "norm": {"eps": 1e-6},
         "layers": [
-            {"type": "parallel", "mixer": _parallel(_attention(3, 3, 10, 14, 0.3), _rot(10, 500.0), (5, 6, 6, 15.0), 1.0, 0.5), "mlp": _moe(12, 4, 4)},
+            {"type": "parallel", "mixer": _parallel(_attention(3, 3, 10, 14, 0.3), _rot(10, 500.0), (5, 6, 6, 18.0), 1.0, 0.4), "mlp": _moe(12, 4, 4)},
             {"type": "channel_delta", "mixer": _delta(3, 3, 10, 14, 1, 3, 9), "mlp": None},
             {"type": "attention", "mixer": _attention(2, 1, 12, 20, 0.35), "mlp": _moe(20, 9, 2, 3.0, (3, 1))},
         ],
@@ -90,7 +90,7 @@ CASES = {
         "architecture": "Natatar", "vocab": 320, "width": 128, "norm": {"eps": 1e-5}, "residual_mult": 0.8,
         "embedding": {"scale": 2.0}, "streams": 4,
         "layers": [
-            {"type": "parallel", "mixer": _parallel(_attention(4, 2, 64, 64, 0.125), _rot(64, 250000.0, (8.0, 32, 8.0, 1.0)), (2, 64, 32, 12.0), 0.9, 0.6),
+            {"type": "parallel", "mixer": _parallel(_attention(4, 2, 64, 64, 0.125), _rot(64, 300000.0, (6.0, 32, 8.0, 1.5)), (2, 64, 32, 12.0), 0.9, 0.6),
              "mlp": _moe(64, 8, 2, 1.25, (4, 3))},
             {"type": "attention", "mixer": _attention(8, 2, 32, 32, 0.18, v_mix=True), "mlp": _moe(32, 4, 2, 1.0, (2, 2))},
             {"type": "channel_delta", "mixer": _delta(2, 2, 128, 64, 2, 8, 8), "mlp": None},

@@ -96,6 +96,7 @@ def test_what_the_configuration_refuses_and_completes():
         (lambda r: r["layers"][3]["mixer"]["left"]["rot"].update(dims=34), "rot"),
         (lambda r: r["layers"][3]["mixer"]["right"].update(gate_cap=0.0), "gate_cap"),
         (lambda r: r["layers"][4]["mixer"].update(vdim=8), "mix values"),
+        (lambda r: r["layers"][4]["mixer"].update(vdim=12, kv_heads=3, heads=3), "mix values"),
         (lambda r: r["layers"][0]["mlp"]["router"]["groups"].update(count=4), "groups"),
         (lambda r: r["layers"][0]["mlp"]["router"]["groups"].update(keep=1, count=6), "groups"),
         (lambda r: r["layers"][1]["mixer"].update(heads=3), "kv_heads"),
@@ -145,9 +146,9 @@ def test_one_stream_with_unit_coefficients_is_the_plain_residual_sum():
 def test_streams_write_from_the_old_streams_all_at_once():
     xs = torch.randn(3, 4, 5, dtype=F)
     M, c, y = torch.randn(3, 3, dtype=F), torch.randn(3, dtype=F), torch.randn(4, 5, dtype=F)
-    new = plain.streams_write(xs, M, c, 0.7, y)
+    new = plain.streams_write(xs, M, c, 0.45, y)
     for r in range(3):
-        want = sum(M[s, r] * xs[s] for s in range(3)) + 0.7 * c[r] * y
+        want = sum(M[s, r] * xs[s] for s in range(3)) + 0.45 * c[r] * y
         assert torch.allclose(new[r], want)
     assert torch.allclose(plain.streams_read(xs, c), sum(c[s] * xs[s] for s in range(3)))
 

@@ -390,7 +390,7 @@ ATTENTIONS = [
     (3, 3, 8, 8, True, None, False),
     (8, 2, 32, 32, True, None, False),
     (2, 1, 128, 64, True, None, False),
-    (6, 3, 96, 96, False, (96, 250000.0, (8.0, 32, 8.0, 1.0)), True),
+    (6, 3, 96, 96, False, (96, 300000.0, (6.0, 32, 8.0, 1.5)), True),
     (2, 1, 32, 16, False, (16, 10000.0, (4.0, 64, 16.0, 2.0)), True),
     (3, 3, 10, 14, False, (10, 500.0, None), True),
     (4, 1, 64, 64, False, (2, 50.0, None), False),
@@ -435,7 +435,7 @@ def test_values_mixed_with_the_first_layers(dtype):
     hidden, T = 48, 40
     gen = torch.Generator().manual_seed(3)
     shapes = [{"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.25, "v_mix": True},
-              {"heads": 2, "kv_heads": 2, "dim": 8, "vdim": 24, "scale": 0.35, "v_mix": True},
+              {"heads": 4, "kv_heads": 4, "dim": 8, "vdim": 12, "scale": 0.35, "v_mix": True},  # other heads, the same projection size
               {"heads": 6, "kv_heads": 2, "dim": 32, "vdim": 24, "scale": 0.18, "v_mix": True}]  # fmt: skip
     ws = [attention_weights(hidden, m, gen, True, False) for m in shapes]
     ws[2]["vmix"] = bf(torch.tensor(0.8))
@@ -515,7 +515,7 @@ def bind_memory(w, hidden, m, dtype, scale=1.0):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", [(3, 8, 24, 10.0), (1, 80, 8, 5.0), (2, 64, 64, 15.0), (2, 200, 16, 30.0), (4, 48, 48, 15.0), (5, 6, 6, 2.0)])
+@pytest.mark.parametrize("shape", [(3, 8, 24, 10.0), (1, 80, 8, 5.0), (2, 64, 64, 18.0), (2, 200, 16, 30.0), (4, 40, 56, 12.0), (5, 6, 6, 2.0)])
 def test_matrix_memory_alone(shape, dtype):
     """Heads and widths of several kinds (keys wider than a lane's slice, values narrower than a wave's columns, a cap
     that the gates reach); the request is cut in rows of 1 to 19 tokens on a slot another request used."""
@@ -743,8 +743,8 @@ def test_streams_are_written_read_and_normed_in_one_pass(sizes, dtype):
     want = plain.rms(plain.streams_read(ref_xs, in_c.double()), 1e-5) * gain.double()
     assert (h.float().cpu() - want).abs().max() <= tol * float(want.abs().max())
     # a pending write, the next read and its norm
-    ops.streams_step(xs, y=y.to(DEV).to(dt), mix=mix.to(DEV), out_c=out_c.to(DEV), mult=0.7, in_c=in_c.to(DEV), gain=gain.to(DEV), eps=1e-5, normed=h)
-    ref_xs = plain.streams_write(ref_xs, mix.double(), out_c.double(), 0.7, y.double())
+    ops.streams_step(xs, y=y.to(DEV).to(dt), mix=mix.to(DEV), out_c=out_c.to(DEV), mult=0.45, in_c=in_c.to(DEV), gain=gain.to(DEV), eps=1e-5, normed=h)
+    ref_xs = plain.streams_write(ref_xs, mix.double(), out_c.double(), 0.45, y.double())
     assert (xs.cpu().double().transpose(0, 1) - ref_xs).abs().max() <= 1e-5 * float(ref_xs.abs().max())
     want = plain.rms(plain.streams_read(ref_xs, in_c.double()), 1e-5) * gain.double()
     assert (h.float().cpu() - want).abs().max() <= tol * float(want.abs().max())
