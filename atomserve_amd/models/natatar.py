@@ -143,9 +143,11 @@ def checkpoint_map(c: NatatarConfig) -> dict:
 
 
 def ignored(c: NatatarConfig) -> set:
-    """The first value-mixing layer's own mixing weight is stored and unused."""
+    """A mixing weight that an attention layer stores and does not use: the first value-mixing layer's own, and that of
+    a layer that mixes nothing."""
     first_mix = _first_mixing_layer(c)
-    return {f"l{first_mix}.mix.vmix"} if first_mix >= 0 else set()
+    return {f"l{i}.mix.vmix" for i, layer in enumerate(c.layers)
+            if layer.type == "attention" and (i == first_mix or not layer.mixer.v_mix)}  # fmt: skip
 
 
 def checkpoint_shapes(c: NatatarConfig) -> dict:
